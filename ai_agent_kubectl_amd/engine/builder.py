@@ -67,7 +67,7 @@ def build_engine(opts: EngineOptions, comm=None, metrics=None) -> LLMEngine:
     dev = torch.device(opts.device)
     if dev.type == "cuda":
         # fail loudly: the GPU path never runs without the HIP kernels of the model's family
-        if getattr(cfg, "family", "llama") in ("vivepel", "kafilorn"):
+        if getattr(cfg, "family", "llama") in ("vivepel", "kafilorn", "suvapel"):
             from ..ops._hip import require_mixers
             require_mixers()
         else:
@@ -80,7 +80,7 @@ def build_engine(opts: EngineOptions, comm=None, metrics=None) -> LLMEngine:
     family = getattr(cfg, "family", "llama")
     if dtype == torch.float32 and family in ("llama", "mixtral"):
         raise ValueError("the Llama / Mixtral kernels are bf16; float32 is served by the fp32-residual families "
-                         "(vivepel, kafilorn)")
+                         "(vivepel, kafilorn, suvapel)")
     if dtype == torch.float32:   # true fp32 products: no reduced-precision matrix mode
         torch.backends.cuda.matmul.allow_tf32 = False
         torch.backends.cudnn.allow_tf32 = False

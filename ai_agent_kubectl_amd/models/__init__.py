@@ -12,4 +12,7 @@ def model_class(cfg):
     if family == "kafilorn":
         from .kafilorn import KafilornModel
         return KafilornModel
+    if family == "suvapel":
+        from .suvapel import SuvapelModel
+        return SuvapelModel
     raise ValueError(f"no model class for family {family!r}")

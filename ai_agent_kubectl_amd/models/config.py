@@ -407,8 +407,265 @@ def kafilorn_uniform(name: str, blocks: int, hidden: int, heads: int, vocab: int
     return KafilornConfig(name, vocab, hidden, 1e-6, streams, 1.0, 1.0, tuple(layers))
 
 
+# ------------------------------------------------------------------------------------------------
+# Suvapel: layers listed one by one; one Dynamic-Tanh norm per layer whose output feeds the mixer and the
+# feed-forward side by side; a layer's mixer is a gated delta rule (recurrent matrix memory with short
+# convolutions, state slots) or that beside sliding-window attention (short convolutions, YaRN-scaled rotary
+# positions, kept first tokens, per-head output gate); a gated feed-forward with biases or none; after it a
+# per-layer token input from a second embedding table.
+@dataclasses.dataclass(frozen=True)
+class RotarySpec:
+    """Rotary positions on the first `dims` entries of a head, pairs (i, i + dims/2), frequency base^(-2i/dims);
+    factor > 0: YaRN scaling (frequencies below the `slow` turn count over `original` positions divided by
+    `factor`, above `fast` kept, a linear ramp between; cos and sin scaled by 0.1 ln(factor) + 1)."""
+    dims: int = 0
+    base: float = 10000.0
+    factor: float = 0.0
+    original: int = 0
+    fast: float = 32.0
+    slow: float = 1.0
+
+    @classmethod
+    def from_dict(cls, rot: Optional[dict]) -> "RotarySpec":
+        if not rot:
+            return cls()
+        sc = rot.get("scaling")
+        if not sc:
+            return cls(int(rot["dims"]), float(rot["base"]))
+        return cls(int(rot["dims"]), float(rot["base"]), float(sc["factor"]), int(sc["original"]), float(sc["fast"]),
+                   float(sc["slow"]))
+
+    def to_dict(self) -> Optional[dict]:
+        if not self.dims:
+            return None
+        d = {"dims": self.dims, "base": self.base}
+        if self.factor > 0:
+            d["scaling"] = {"factor": self.factor, "original": self.original, "fast": self.fast, "slow": self.slow}
+        return d
+
+    def frequencies(self):
+        """(frequencies [dims / 2] as float64 list, magnitude factor of cos and sin)."""
+        import math
+
+        half = self.dims // 2
+        f = [float(self.base) ** (-2.0 * i / self.dims) for i in range(half)]
+        if self.factor <= 0 or half == 0:
+            return f, 1.0
+
+        def turn_dim(turns: float) -> float:
+            return self.dims * math.log(self.original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.base))
+
+        lo = max(math.floor(turn_dim(self.fast)), 0)
+        hi = min(math.ceil(turn_dim(self.slow)), self.dims - 1)
+        out = []
+        for i in range(half):
+            ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            out.append(f[i] / self.factor * ramp + f[i] * (1.0 - ramp))
+        return out, 0.1 * math.log(self.factor) + 1.0
+
+
+@dataclasses.dataclass(frozen=True)
+class SlidingAttentionSpec:
+    """Softmax attention with grouped keys / values, a short causal convolution on q, k and v, rotary positions,
+    a sliding window that also keeps the sequence's first tokens, and a sigmoid gate per head on the output."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int                   # taps of the short convolution (1: none)
+    window: int                 # position i sees j <= i with i - j < window (0: all) ...
+    keep_first: int             # ... or j < keep_first
+    rot: RotarySpec
+    scale: float
+    kind: str = "sliding_attention"
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "SlidingAttentionSpec":
+        mask = m.get("mask") or {}
+        spec = cls(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                   conv=int(m.get("conv") or 1), window=int(mask.get("size") or 0), keep_first=int(mask.get("keep_first") or 0),
+                   rot=RotarySpec.from_dict(m.get("rot")), scale=float(m["scale"]))
+        if spec.heads % spec.kv_heads or spec.conv < 1 or spec.window < 0 or spec.keep_first < 0:
+            raise ValueError(f"bad attention sizes: {spec}")
+        if spec.rot.dims % 2 or spec.rot.dims > spec.dim:
+            raise ValueError(f"bad rotary dims {spec.rot.dims} for head size {spec.dim}")
+        return spec
+
+    def to_dict(self) -> dict:
+        d = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "conv": self.conv,
+             "scale": self.scale}
+        if self.window or self.keep_first:
+            d["mask"] = {"size": self.window, "keep_first": self.keep_first}
+        if self.rot.dims:
+            d["rot"] = self.rot.to_dict()
+        return d
+
+
+@dataclasses.dataclass(frozen=True)
+class DeltaSpec:
+    """Gated delta rule: per head a [dim, vdim] memory that is decayed, corrected towards the value along the
+    unit key, and read with the query; q / k come in kv_heads groups.  channel_decay: one decay per head and key
+    channel (through a low-rank pair, with a sigmoid low-rank output gate) instead of one per head (silu gate).
+    low_rank: the inner size of those pairs when weights are drawn at random; a checkpoint's tensors give theirs."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    channel_decay: bool = False
+    low_rank: int = 16
+    kind: str = "delta"
+
+    @classmethod
+    def from_dict(cls, m: dict, channel_decay: bool = False) -> "DeltaSpec":
+        spec = cls(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                   conv=int(m.get("conv") or 1), channel_decay=channel_decay)
+        if spec.heads % spec.kv_heads or spec.conv < 1:
+            raise ValueError(f"bad delta-rule sizes: {spec}")
+        return spec
+
+    def to_dict(self) -> dict:
+        return {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "conv": self.conv}
+
+    def state_floats(self) -> int:
+        return self.heads * self.dim * self.vdim
+
+    def conv_channels(self) -> int:
+        return 2 * self.kv_heads * self.dim + self.heads * self.vdim
+
+
+@dataclasses.dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Attention and a delta rule side by side on the same input: left_scale * left + right_scale * right."""
+    left: SlidingAttentionSpec
+    right: DeltaSpec
+    left_scale: float
+    right_scale: float
+    kind: str = "parallel"
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "ParallelMixerSpec":
+        return cls(SlidingAttentionSpec.from_dict(m["left"]), DeltaSpec.from_dict(m["right"], channel_decay=True),
+                   float(m["left_scale"]), float(m["right_scale"]))
+
+    def to_dict(self) -> dict:
+        return {"left": self.left.to_dict(), "right": self.right.to_dict(), "left_scale": self.left_scale,
+                "right_scale": self.right_scale}
+
+
+@dataclasses.dataclass(frozen=True)
+class SuvapelLayer:
+    mixer: object               # DeltaSpec | ParallelMixerSpec
+    ff: int = 0                 # width of the gated feed-forward; 0: none
+
+    @property
+    def delta(self) -> DeltaSpec:
+        return self.mixer.right if self.mixer.kind == "parallel" else self.mixer
+
+    @property
+    def attention(self) -> Optional[SlidingAttentionSpec]:
+        return self.mixer.left if self.mixer.kind == "parallel" else None
+
+
+@dataclasses.dataclass(frozen=True)
+class SuvapelConfig:
+    name: str
+    vocab_size: int
+    hidden: int
+    norm_eps: float
+    residual_mult: float        # every sublayer result enters the residual times this
+    side_dim: int               # per-layer slice of the second embedding table; 0: no token input
+    layers: Tuple[SuvapelLayer, ...]
+    max_position: int = 1 << 20
+    tokenizer: str = "llama3"
+    family: str = "suvapel"
+    tie_embeddings: bool = False
+    is_moe: bool = False
+    has_state: bool = True
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_dict(cls, d: dict, name: str = "suvapel") -> "SuvapelConfig":
+        layers = []
+        for i, L in enumerate(d["layers"]):
+            if L["type"] == "delta":
+                mixer = DeltaSpec.from_dict(L["mixer"])
+            elif L["type"] == "parallel":
+                mixer = ParallelMixerSpec.from_dict(L["mixer"])
+            else:
+                raise ValueError(f"layer {i}: unknown mixer type {L['type']!r}")
+            mlp = L.get("mlp")
+            if mlp is not None and mlp.get("kind") != "dense":
+                raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+            layers.append(SuvapelLayer(mixer, int(mlp["ff"]) if mlp is not None else 0))
+        side = d.get("token_side") or {}
+        return cls(name=name, vocab_size=int(d["vocab"]), hidden=int(d["width"]), norm_eps=float(d["norm"]["eps"]),
+                   residual_mult=float(d.get("residual_mult", 1.0)), side_dim=int(side.get("dim") or 0), layers=tuple(layers))
+
+    def to_dict(self) -> dict:
+        d = {"architecture": "Suvapel", "vocab": self.vocab_size, "width": self.hidden, "norm": {"eps": self.norm_eps},
+             "residual_mult": self.residual_mult,
+             "layers": [{"type": L.mixer.kind, "mixer": L.mixer.to_dict(),
+                         "mlp": {"kind": "dense", "ff": L.ff} if L.ff else None} for L in self.layers]}
+        if self.side_dim:
+            d["token_side"] = {"dim": self.side_dim}
+        return d
+
+    def num_params(self) -> int:
+        h = self.hidden
+        n = 2 * self.vocab_size * h + 2 * h + 1 + self.vocab_size * self.side_dim * len(self.layers)
+        for L in self.layers:
+            m, a = L.delta, L.attention
+            n += h * (m.conv_channels() + m.heads) + m.conv_channels() * m.conv + m.heads * m.vdim * h + 2 * m.heads + m.vdim
+            if m.channel_decay:
+                n += 2 * m.low_rank * h + m.low_rank * m.heads * (m.dim + m.vdim) + m.heads * m.dim
+            else:
+                n += h * m.heads * (1 + m.vdim)
+            if a is not None:
+                c = a.heads * a.dim + a.kv_heads * (a.dim + a.vdim)
+                n += c * (h + a.conv) + a.heads * h + a.heads * a.vdim * h
+            if L.ff:
+                n += 3 * h * L.ff + 2 * L.ff + h
+            n += 2 * h + 1 + (2 * self.side_dim * h + h if self.side_dim else 0)
+        return n
+
+    def default_step_tokens(self) -> int:
+        return 8192
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        """Paged cache per token: keys and values of every attention half."""
+        return max(1, sum(L.attention.kv_heads * (L.attention.dim + L.attention.vdim) * dtype_bytes
+                          for L in self.layers if L.attention is not None))
+
+    def state_bytes_per_slot(self, dtype_bytes: int = 2) -> int:
+        """Per sequence slot: the delta-rule memories (fp32) and the convolutions' last inputs."""
+        n = 0
+        for L in self.layers:
+            m, a = L.delta, L.attention
+            n += m.state_floats() * 4 + (m.conv - 1) * m.conv_channels() * dtype_bytes
+            if a is not None:
+                n += (a.conv - 1) * (a.heads * a.dim + a.kv_heads * (a.dim + a.vdim)) * dtype_bytes
+        return n
+
+
+def suvapel_uniform(name: str, layers: int, hidden: int, heads: int, kv_heads: int, dim: int, ff: int, vocab: int,
+                    window: int = 1024, keep_first: int = 4, side_dim: int = 64, conv: int = 4, every: int = 2,
+                    low_rank: int = 64) -> SuvapelConfig:
+    """A regular Suvapel (benchmarks, tests): every `every`-th layer a plain delta layer, the others attention
+    beside a channel-decay delta rule; all heads of size dim."""
+    rot = RotarySpec(dim // 2, 10000.0, 8.0, 4096, 32.0, 1.0)
+    att = SlidingAttentionSpec(heads, kv_heads, dim, dim, conv, window, keep_first, rot, dim ** -0.5)
+    plain = DeltaSpec(heads, kv_heads, dim, dim, conv, False, low_rank)
+    par = ParallelMixerSpec(att, DeltaSpec(heads, kv_heads, dim, dim, conv, True, low_rank), 0.5, 0.5)
+    ls = tuple(SuvapelLayer(plain if every and i % every == 0 else par, ff) for i in range(layers))
+    return SuvapelConfig(name, vocab, hidden, 1e-5, 1.0, side_dim, ls)
+
+
 # config.json "architecture" -> parser of the file's dict
-ARCHITECTURES = {"Vivepel": VivepelConfig.from_dict, "Kafilorn": KafilornConfig.from_dict}
+ARCHITECTURES = {"Vivepel": VivepelConfig.from_dict, "Kafilorn": KafilornConfig.from_dict, "Suvapel": SuvapelConfig.from_dict}
 
 
 def load_config_dir(path: str):
@@ -451,6 +708,10 @@ PRESETS: Dict[str, ModelConfig] = {
                                       streams=2, kv_rank=48, q_rank=40, dim=24, rot_dim=8),
     "kafilorn-4k-3l": kafilorn_uniform("kafilorn-4k-3l", 1, 4096, 32, 128256, 14336, experts=8, top=2, expert_ff=3584,
                                        window=1024, streams=2, kv_rank=512, q_rank=1536, dim=128, rot_dim=64),
+    # Suvapel at a small size (CPU tests) and at a Llama-3-8B-like width (bench.py --arch-compare)
+    "tiny-suvapel": suvapel_uniform("tiny-suvapel", 3, 128, 4, 2, 32, 192, 384, window=24, keep_first=3, side_dim=16,
+                                    conv=3, every=3, low_rank=8),
+    "suvapel-4k-2l": suvapel_uniform("suvapel-4k-2l", 2, 4096, 32, 8, 128, 14336, 128256),
 }
 
 

@@ -491,6 +491,202 @@ def load_kafilorn_safetensors(path: str, cfg, device="cpu", dtype=torch.bfloat16
     return W
 
 
+# ------------------------------------------------------------------------------------------------
+# Suvapel.  Engine layout per layer `layers.<i>.` (activation dtype unless marked fp32):
+#   norm_w, norm_b [W], norm_alpha [1]                                                         fp32
+#   w_in [P, W]: every projection that reads the layer's normed row, stacked for one GEMM, each segment padded
+#           with zero rows to a multiple of 8 columns (`suvapel_columns`): attention q | k | v | head gates,
+#           delta q | k | v | beta | decay (per head, or the low-rank pair's first half) | output gate (full, or the
+#           low-rank pair's first half), feed-forward gate | up
+#   att_conv [q + k + v channels, taps], conv [q + k + v channels, taps]                        fp32
+#   inv_freq [rot dims / 2] fp32 (YaRN-scaled, float64 rounded once), att_wo [W, H * Dv]
+#   A_log [H], dt_bias [H] or [H * D], hnorm [H * Dv] (the shared [Dv] weight repeated per head)  fp32
+#   w_a2 [H * D, R], w_g2 [H * Dv, R] (channel decay only), wo [W, H * Dv]
+#   b_gu [2 ff] fp32, w_down [W, ff], b_down [W]
+#   side_gate [dim, W], side_proj [W, dim], side_norm [W] fp32
+# Global: embed, lm_head, side_embed [V, L * dim], norm_w / norm_b / norm_alpha (the final norm).
+_SUVAPEL_F32 = ("norm_w", "norm_b", "norm_alpha", "att_conv", "conv", "inv_freq", "A_log", "dt_bias", "hnorm", "b_gu",
+                "side_norm")
+
+
+def _pad8(n: int) -> int:
+    return (n + 7) // 8 * 8
+
+
+def suvapel_columns(L, rank_a: int = 0, rank_g: int = 0) -> Dict[str, int]:
+    """Column offsets of a layer's fused input projection (segment name -> first column; "total": the row length).
+    rank_a / rank_g: inner sizes of the channel-decay and output-gate pairs (ignored for a per-head decay)."""
+    col, o = {}, 0
+
+    def seg(name, n):
+        nonlocal o
+        col[name] = o
+        o += _pad8(n)
+
+    a, m = L.attention, L.delta
+    if a is not None:
+        seg("att_q", a.heads * a.dim + a.kv_heads * (a.dim + a.vdim))   # q | k | v contiguous: one convolution
+        seg("att_g", a.heads)
+    seg("q", m.conv_channels())                                         # q | k | v contiguous
+    seg("beta", m.heads)
+    seg("a", rank_a if m.channel_decay else m.heads)
+    seg("g", rank_g if m.channel_decay else m.heads * m.vdim)
+    if L.ff:
+        seg("ff", 2 * L.ff)                                             # gate | up contiguous
+    col["total"] = o
+    return col
+
+
+def _suvapel_pack(cfg, get, device, dtype) -> Dict[str, torch.Tensor]:
+    h = cfg.hidden
+    W: Dict[str, torch.Tensor] = {"embed": get("embed"), "lm_head": get("head"), "norm_w": get("final.norm"),
+                                  "norm_b": get("final.norm.b"), "norm_alpha": get("final.norm.alpha").reshape(1)}
+    if cfg.side_dim:
+        W["side_embed"] = get("side.embed")
+    for i, L in enumerate(cfg.layers):
+        p, c, m, a = f"layers.{i}.", f"l{i}.", L.delta, L.attention
+        W[p + "norm_w"], W[p + "norm_b"] = get(c + "norm1"), get(c + "norm1.b")
+        W[p + "norm_alpha"] = get(c + "norm1.alpha").reshape(1)
+        r = c + ("mix.right." if a is not None else "mix.")
+        rank_a = get(r + "a1").shape[0] if m.channel_decay else 0
+        rank_g = get(r + "g1").shape[0] if m.channel_decay else 0
+        col = suvapel_columns(L, rank_a, rank_g)
+        w_in = torch.zeros((col["total"], h), dtype=get(r + "q").dtype)
+
+        def put(name, *tensors):
+            t = torch.cat(tensors)
+            w_in[col[name]:col[name] + t.shape[0]] = t
+
+        if a is not None:
+            l = c + "mix.left."
+            put("att_q", get(l + "q"), get(l + "k"), get(l + "v"))
+            put("att_g", get(l + "g"))
+            W[p + "att_conv"] = torch.cat([get(l + "q.conv"), get(l + "k.conv"), get(l + "v.conv")])
+            W[p + "att_wo"] = get(l + "o")
+            W[p + "inv_freq"] = torch.tensor(a.rot.frequencies()[0], dtype=torch.float64)
+        put("q", get(r + "q"), get(r + "k"), get(r + "v"))
+        put("beta", get(r + "b"))
+        put("a", get(r + "a1") if m.channel_decay else get(r + "a"))
+        put("g", get(r + "g1") if m.channel_decay else get(r + "g"))
+        W[p + "conv"] = torch.cat([get(r + "q.conv"), get(r + "k.conv"), get(r + "v.conv")])
+        W[p + "A_log"], W[p + "dt_bias"] = get(r + "A_log"), get(r + "dt_bias")
+        W[p + "hnorm"] = get(r + "norm").repeat(m.heads)
+        if m.channel_decay:
+            W[p + "w_a2"], W[p + "w_g2"] = get(r + "a2"), get(r + "g2")
+        W[p + "wo"] = get(r + "o")
+        if L.ff:
+            put("ff", get(c + "mlp.gate"), get(c + "mlp.up"))
+            W[p + "b_gu"] = torch.cat([get(c + "mlp.gate.b"), get(c + "mlp.up.b")])
+            W[p + "w_down"], W[p + "b_down"] = get(c + "mlp.down"), get(c + "mlp.down.b")
+        if cfg.side_dim:
+            W[p + "side_gate"], W[p + "side_proj"], W[p + "side_norm"] = get(c + "side.gate"), get(c + "side.proj"), get(c + "side.norm")
+        W[p + "w_in"] = w_in
+    out = {}
+    for k, v in W.items():
+        f32 = k.rsplit(".", 1)[-1] in _SUVAPEL_F32
+        out[k] = v.to(device=device, dtype=torch.float32 if f32 else dtype).contiguous()
+    return out
+
+
+def suvapel_check_shapes(cfg, W: Dict[str, torch.Tensor]) -> None:
+    """Every tensor of the engine layout has the shape the configuration implies (the low-rank pairs' inner sizes
+    are the tensors' own)."""
+    h, V = cfg.hidden, cfg.vocab_size
+    want = {"embed": (V, h), "lm_head": (V, h), "norm_w": (h,), "norm_b": (h,), "norm_alpha": (1,)}
+    if cfg.side_dim:
+        want["side_embed"] = (V, cfg.side_dim * cfg.num_layers)
+    for i, L in enumerate(cfg.layers):
+        p, m, a = f"layers.{i}.", L.delta, L.attention
+        ra = W[p + "w_a2"].shape[1] if p + "w_a2" in W else 0
+        rg = W[p + "w_g2"].shape[1] if p + "w_g2" in W else 0
+        want.update({p + "norm_w": (h,), p + "norm_b": (h,), p + "norm_alpha": (1,),
+                     p + "w_in": (suvapel_columns(L, ra, rg)["total"], h), p + "conv": (m.conv_channels(), m.conv),
+                     p + "A_log": (m.heads,), p + "dt_bias": (m.heads * m.dim if m.channel_decay else m.heads,),
+                     p + "hnorm": (m.heads * m.vdim,), p + "wo": (h, m.heads * m.vdim)})
+        if m.channel_decay:
+            want.update({p + "w_a2": (m.heads * m.dim, ra), p + "w_g2": (m.heads * m.vdim, rg)})
+        if a is not None:
+            want.update({p + "att_conv": (a.heads * a.dim + a.kv_heads * (a.dim + a.vdim), a.conv),
+                         p + "att_wo": (h, a.heads * a.vdim), p + "inv_freq": (a.rot.dims // 2,)})
+        if L.ff:
+            want.update({p + "b_gu": (2 * L.ff,), p + "w_down": (h, L.ff), p + "b_down": (h,)})
+        if cfg.side_dim:
+            want.update({p + "side_gate": (cfg.side_dim, h), p + "side_proj": (h, cfg.side_dim), p + "side_norm": (h,)})
+    for k, shp in want.items():
+        if k not in W or tuple(W[k].shape) != shp:
+            raise ValueError(f"tensor {k}: expected shape {shp}, found {tuple(W[k].shape) if k in W else None}")
+
+
+def suvapel_checkpoint_tensors(cfg, seed: int = 0, dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Random tensors under the checkpoint's own names (what a Suvapel model.safetensors holds)."""
+    g = torch.Generator().manual_seed(_seed(seed, "suvapel") & 0x7FFFFFFF)
+    h, V = cfg.hidden, cfg.vocab_size
+
+    def mat(o, i, std=None):
+        return (torch.randn(o, i, generator=g) * (std if std is not None else i ** -0.5)).to(dtype)
+
+    def vec(n, lo=0.75, hi=1.25):
+        return (lo + (hi - lo) * torch.rand(n, generator=g)).to(dtype)
+
+    def dyt(name):
+        return {name: vec(h), name + ".b": (torch.randn(h, generator=g) * 0.05).to(dtype),
+                name + ".alpha": (0.4 + 0.4 * torch.rand((), generator=g)).to(dtype)}
+
+    def conv(c, taps):
+        w = torch.randn(c, taps, generator=g) * 0.3
+        w[:, -1] += 1.0
+        return w.to(dtype)
+
+    T = {"embed": mat(V, h, 1.0), "head": mat(V, h), **dyt("final.norm")}
+    if cfg.side_dim:
+        T["side.embed"] = mat(V, cfg.side_dim * cfg.num_layers, 1.0)
+    for i, L in enumerate(cfg.layers):
+        c, m, a = f"l{i}.", L.delta, L.attention
+        T.update(dyt(c + "norm1"))
+        if a is not None:
+            l = c + "mix.left."
+            for k, n in (("q", a.heads * a.dim), ("k", a.kv_heads * a.dim), ("v", a.kv_heads * a.vdim)):
+                T[l + k], T[l + k + ".conv"] = mat(n, h), conv(n, a.conv)
+            T[l + "g"], T[l + "o"] = mat(a.heads, h), mat(h, a.heads * a.vdim)
+        r = c + ("mix.right." if a is not None else "mix.")
+        for k, n in (("q", m.kv_heads * m.dim), ("k", m.kv_heads * m.dim), ("v", m.heads * m.vdim)):
+            T[r + k], T[r + k + ".conv"] = mat(n, h, 2.0 * h ** -0.5), conv(n, m.conv)
+        T[r + "b"] = mat(m.heads, h)
+        T[r + "A_log"] = torch.log(0.5 + 3.5 * torch.rand(m.heads, generator=g)).to(dtype)
+        T[r + "norm"], T[r + "o"] = vec(m.vdim), mat(h, m.heads * m.vdim)
+        if m.channel_decay:
+            R = m.low_rank
+            T[r + "a1"], T[r + "a2"] = mat(R, h), mat(m.heads * m.dim, R)
+            T[r + "g1"], T[r + "g2"] = mat(R, h), mat(m.heads * m.vdim, R)
+            T[r + "dt_bias"] = (torch.randn(m.heads * m.dim, generator=g) - 3.0).to(dtype)
+        else:
+            T[r + "a"], T[r + "g"] = mat(m.heads, h), mat(m.heads * m.vdim, h)
+            T[r + "dt_bias"] = (torch.randn(m.heads, generator=g) - 3.0).to(dtype)
+        if L.ff:
+            for k, o_, i_ in (("gate", L.ff, h), ("up", L.ff, h), ("down", h, L.ff)):
+                T[c + "mlp." + k] = mat(o_, i_)
+                T[c + "mlp." + k + ".b"] = (torch.randn(o_, generator=g) * 0.1).to(dtype)
+        if cfg.side_dim:
+            T[c + "side.gate"], T[c + "side.proj"] = mat(cfg.side_dim, h), mat(h, cfg.side_dim)
+            T[c + "side.norm"] = vec(h, 0.2, 0.6)
+    return T
+
+
+def suvapel_random_weights(cfg, seed: int = 0, device="cpu", dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Random-init Suvapel weights: drawn in bf16 (as a checkpoint stores them), packed for `dtype`."""
+    T = suvapel_checkpoint_tensors(cfg, seed)
+    W = _suvapel_pack(cfg, T.__getitem__, device, dtype)
+    suvapel_check_shapes(cfg, W)
+    return W
+
+
+def load_suvapel_safetensors(path: str, cfg, device="cpu", dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """A Suvapel checkpoint (a file, or a folder holding model.safetensors / *.safetensors)."""
+    W = _suvapel_pack(cfg, _safetensors_getter(path), device, dtype)
+    suvapel_check_shapes(cfg, W)
+    return W
+
+
 def build_weights(spec: str, cfg: ModelConfig, par: ParallelInfo, device="cpu", dtype=torch.bfloat16):
     if getattr(cfg, "family", "") == "vivepel":
         if par.tp_size != 1 or par.ep_size != 1:
@@ -506,6 +702,13 @@ def build_weights(spec: str, cfg: ModelConfig, par: ParallelInfo, device="cpu", 
             seed = int(spec.split(":", 1)[1]) if ":" in spec else 0
             return kafilorn_random_weights(cfg, seed=seed, device=device, dtype=dtype)
         return load_kafilorn_safetensors(spec, cfg, device=device, dtype=dtype)
+    if getattr(cfg, "family", "") == "suvapel":
+        if par.tp_size != 1 or par.ep_size != 1:
+            raise ValueError("Suvapel runs at TP = 1 (data parallel replicas scale it out)")
+        if spec.startswith("random"):
+            seed = int(spec.split(":", 1)[1]) if ":" in spec else 0
+            return suvapel_random_weights(cfg, seed=seed, device=device, dtype=dtype)
+        return load_suvapel_safetensors(spec, cfg, device=device, dtype=dtype)
     if spec.startswith("random"):
         seed = int(spec.split(":", 1)[1]) if ":" in spec else 0
         return random_weights(cfg, par, seed=seed, device=device, dtype=dtype)

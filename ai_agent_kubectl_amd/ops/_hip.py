@@ -120,7 +120,7 @@ _MIX_SIGS = {
     "ka_stream_update": [P, P, P, P, P, P, P, I, I, I, F, I, I, P],
     "ka_relu_sq": [P, P, ctypes.c_long, I, P],
     "ka_silu_mul_rows": [P, P, I, I, I, P],
-    "ka_headnorm_gate": [P, P, P, P, I, I, P, I, I, I, F, I, P],
+    "ka_headnorm_gate": [P, P, P, P, I, I, P, I, I, I, F, I, I, P],
     "ka_mlstm_gates": [P, P, P, P, I, I, I, F, I, P],
     "ka_mlstm_gates_mfma": [P, P, P, P, I, I, I, F, P],
     "ka_mlstm_scan": [P, P, P, I, I, I, I, P, P, P, P, P, P, P, I, P, I, I, I, F, I, P],
@@ -130,6 +130,16 @@ _MIX_SIGS = {
     "ka_moe_route": [P, P, P, P, P, I, I, I, I, I, I, I, P],
     "ka_moe_rows": [P, P, P, P, P, P, P, I, I, I, I, I, P],
     "ka_moe_grouped": [P, P, P, P, P, P, P, P, I, I, I, I, I, P],
+    "ka_dyt_norm": [P, P, P, P, P, I, I, I, P],
+    "ka_residual_mix": [P, P, P, P, F, F, F, P, P, P, P, P, I, I, I, I, P],
+    "ka_rms_residual": [P, P, P, F, F, P, P, P, P, I, I, I, I, P],
+    "ka_gelu_gate_embed": [P, P, P, P, I, I, I, I, I, I, P],
+    "ka_silu_mul_bias": [P, P, I, I, I, P, I, I, P],
+    "ka_short_conv": [P, P, I, I, I, P, I, P, P, P, I, P, I, I, I, P],
+    "ka_rope_append": [P, P, P, F, P, P, P, P, I, I, I, I, I, I, I, I, P],
+    "ka_sliding_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, I, I, F, I, I, P],
+    "ka_delta_prep": [P, P, P, P, I, P, I, I, P, I, I, P, P, I, I, I, I, I, I, P],
+    "ka_delta_scan": [P, P, P, I, I, P, P, P, P, P, I, P, I, I, I, I, I, I, P],
 }
 MIXERS_LIB = os.path.join(LIB_DIR, "libkagent_mixers.so")
 _mix: Optional[ctypes.CDLL] = None

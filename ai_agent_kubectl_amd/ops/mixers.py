@@ -296,11 +296,11 @@ def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, gates: to
 
 
 def headnorm_gate(o: torch.Tensor, proj: torch.Tensor, g_off: int, w: torch.Tensor, H: int, Dv: int, eps: float,
-                  out_dtype, den: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  out_dtype, den: Optional[torch.Tensor] = None, silu: bool = False) -> torch.Tensor:
     """o [T, H * Dv] fp32 (each head first divided by den [T, H], if given): each head divided by its root mean
-    square, times w, times sigmoid(proj[:, g_off:...])."""
+    square, times w, times sigmoid(proj[:, g_off:...]) (silu: times silu of those columns)."""
     if _ref(o):
-        return ref.headnorm_gate(o, proj, g_off, w, H, Dv, eps, out_dtype, den)
+        return ref.headnorm_gate(o, proj, g_off, w, H, Dv, eps, out_dtype, den, silu)
     lib = require_mixers()
     T = o.shape[0]
     assert o.dtype == torch.float32 and o.is_contiguous() and proj.is_contiguous() and proj.dtype == out_dtype
@@ -308,7 +308,7 @@ def headnorm_gate(o: torch.Tensor, proj: torch.Tensor, g_off: int, w: torch.Tens
     assert den is None or (den.dtype == torch.float32 and den.shape == (T, H) and den.is_contiguous())
     out = torch.empty((T, H * Dv), dtype=out_dtype, device=o.device)
     check(lib.ka_headnorm_gate(_p(out), _p(o), _p(den), _p(proj), proj.shape[1], g_off, _p(w), T, H, Dv, float(eps),
-                               _f32(out), _stream()), "headnorm_gate")
+                               int(bool(silu)), _f32(out), _stream()), "headnorm_gate")
     return out
 
 
@@ -434,4 +434,229 @@ def moe_experts(h: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor, ids: 
             ys[off:off + c] = F.linear(silu_mul(F.linear(xs[off:off + c], w_gu[e])), w_down[e])
             off += c
     out.index_add_(0, tok, ys.float() * w.reshape(-1).index_select(0, order).unsqueeze(1))
+    return out
+
+
+# ------------------------------------------------------------------------------------------------
+# Dynamic-Tanh norm and scaled residual sums (csrc/residual_dyt.hip), short convolutions over state slots
+# (csrc/short_conv.hip), rotary positions from a frequency table + sliding-window attention that keeps the first
+# tokens (csrc/attention_window.hip), the gated delta rule (csrc/delta_rule.hip)
+def _dyt_ok(dyt, width: int) -> None:
+    alpha, w, b = dyt
+    assert alpha.dtype == w.dtype == b.dtype == torch.float32 and alpha.numel() == 1 and w.numel() == b.numel() == width
+
+
+def dyt_norm(x: torch.Tensor, alpha: torch.Tensor, w: torch.Tensor, b: torch.Tensor, out_dtype) -> torch.Tensor:
+    """Dynamic Tanh: tanh(alpha * x) * w + b per entry, no statistics.  x [T, W] fp32, alpha a one-element fp32
+    tensor -> [T, W] in out_dtype."""
+    if _ref(x):
+        return ref.dyt_norm(x, alpha, w, b, out_dtype)
+    lib = require_mixers()
+    T, W = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    _dyt_ok((alpha, w, b), W)
+    out = torch.empty((T, W), dtype=out_dtype, device=x.device)
+    check(lib.ka_dyt_norm(_p(out), _p(x), _p(alpha), _p(w), _p(b), T, W, _f32(out), _stream()), "dyt_norm")
+    return out
+
+
+def residual_mix(x: torch.Tensor, ys, coefs, out_dtype, want_copy: bool = False, dyt=None):
+    """x [T, W] fp32 += sum_i coefs[i] * ys[i] in place (one to three sublayer results in the activation dtype,
+    summed in fp32); returns (x rounded to out_dtype if want_copy, dyt_norm(x, *dyt) if dyt = (alpha, w, b)), both
+    written in the same pass."""
+    assert 1 <= len(ys) <= 3 and len(ys) == len(coefs)
+    if _ref(x):
+        return ref.residual_mix(x, ys, coefs, out_dtype, want_copy, dyt)
+    lib = require_mixers()
+    T, W = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    for y in ys:
+        assert y.shape == (T, W) and y.is_contiguous() and y.dtype == ys[0].dtype
+    if dyt is not None:
+        _dyt_ok(dyt, W)
+    yp = [_p(y) for y in ys] + [None] * (3 - len(ys))
+    cs = [float(c) for c in coefs] + [0.0] * (3 - len(ys))
+    xa = torch.empty((T, W), dtype=out_dtype, device=x.device) if want_copy else None
+    h = torch.empty((T, W), dtype=out_dtype, device=x.device) if dyt is not None else None
+    al, dw, db = dyt if dyt is not None else (None, None, None)
+    check(lib.ka_residual_mix(_p(x), *yp, *cs, _p(xa), _p(h), _p(al), _p(dw), _p(db), T, W, _f32(ys[0]),
+                              1 if out_dtype == torch.float32 else 0, _stream()), "residual_mix")
+    return xa, h
+
+
+def rms_residual(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, mult: float, eps: float, out_dtype, dyt=None):
+    """x [T, W] fp32 += mult * y / sqrt(mean(y^2) + eps) * w in place; returns dyt_norm(x, *dyt) from the same pass
+    (None without dyt)."""
+    if _ref(x):
+        return ref.rms_residual(x, y, w, mult, eps, out_dtype, dyt)
+    lib = require_mixers()
+    T, W = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous() and y.shape == (T, W) and y.is_contiguous()
+    assert w.dtype == torch.float32 and w.numel() == W
+    if dyt is not None:
+        _dyt_ok(dyt, W)
+    h = torch.empty((T, W), dtype=out_dtype, device=x.device) if dyt is not None else None
+    al, dw, db = dyt if dyt is not None else (None, None, None)
+    check(lib.ka_rms_residual(_p(x), _p(y), _p(w), float(mult), float(eps), _p(h), _p(al), _p(dw), _p(db), T, W, _f32(y),
+                              1 if out_dtype == torch.float32 else 0, _stream()), "rms_residual")
+    return h
+
+
+def gelu_gate_embed(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col0: int) -> torch.Tensor:
+    """gelu_tanh(z) * table[ids, col0 : col0 + dim] for z [T, dim]: a gate on a slice of an embedding row."""
+    if _ref(z):
+        return ref.gelu_gate_embed(z, table, ids, col0)
+    lib = require_mixers()
+    T, dim = z.shape
+    assert z.is_contiguous() and table.is_contiguous() and table.dtype == z.dtype and ids.dtype == torch.int32
+    assert 0 <= col0 and col0 + dim <= table.shape[1] and ids.shape[0] >= T
+    out = torch.empty_like(z)
+    check(lib.ka_gelu_gate_embed(_p(out), _p(z), _p(table), _p(ids), T, dim, table.shape[1], col0, table.shape[0], _f32(z),
+                                 _stream()), "gelu_gate_embed")
+    return out
+
+
+def silu_mul_bias(proj: torch.Tensor, off: int, ff: int, bias: torch.Tensor) -> torch.Tensor:
+    """silu(gate + bias[:ff]) * (up + bias[ff:]) with gate | up = proj[:, off : off + 2 ff] -> [T, ff]."""
+    if _ref(proj):
+        return ref.silu_mul_bias(proj, off, ff, bias)
+    lib = require_mixers()
+    T, P = proj.shape
+    assert proj.is_contiguous() and off >= 0 and off + 2 * ff <= P and bias.dtype == torch.float32 and bias.numel() == 2 * ff
+    out = torch.empty((T, ff), dtype=proj.dtype, device=proj.device)
+    check(lib.ka_silu_mul_bias(_p(out), _p(proj), P, off, ff, _p(bias), T, _f32(proj), _stream()), "silu_mul_bias")
+    return out
+
+
+def short_conv(proj: torch.Tensor, off: int, C: int, w: torch.Tensor, state: Optional[torch.Tensor],
+               seq_slots: torch.Tensor, q_starts: Optional[torch.Tensor], positions: torch.Tensor, act: bool) -> torch.Tensor:
+    """A causal convolution over time per channel, y_t = sum_j w[:, j] * u_(t - taps + 1 + j), on the columns
+    u = proj[:, off : off + C] of each sequence's rows.  Inputs from before this step come from state[slot]
+    [taps - 1, C] (the sequence's last inputs, newest last), inputs before position 0 are zero, so a slot needs no
+    clearing; afterwards the state holds the last inputs including this step's.  act: silu on the result.
+    w [C, taps] fp32; state [slots, taps - 1, C] in proj's dtype (None when taps is 1).  q_starts None: row t is
+    sequence t.  -> [T, C]."""
+    taps = w.shape[1]
+    if _ref(proj):
+        return ref.short_conv(proj, off, C, w, state, seq_slots, q_starts, positions, act)
+    lib = require_mixers()
+    T, P = proj.shape
+    nseq = seq_slots.shape[0]
+    assert proj.is_contiguous() and off >= 0 and off + C <= P and w.dtype == torch.float32 and w.shape == (C, taps)
+    assert w.is_contiguous() and seq_slots.dtype == torch.int32 and positions.dtype == torch.int32 and positions.shape[0] >= T
+    assert taps == 1 or (state is not None and state.dtype == proj.dtype and state.shape[1:] == (taps - 1, C)
+                         and state.is_contiguous())
+    assert (q_starts is None and nseq <= T) or (q_starts is not None and q_starts.dtype == torch.int32
+                                                 and q_starts.shape[0] == nseq + 1)
+    out = torch.zeros((T, C), dtype=proj.dtype, device=proj.device)
+    check(lib.ka_short_conv(_p(out), _p(proj), P, off, C, _p(w), taps, _p(state), _p(seq_slots), _p(q_starts), nseq,
+                            _p(positions), T, int(bool(act)), _f32(proj), _stream()), "short_conv")
+    return out
+
+
+def rope_append(qkv: torch.Tensor, inv_freq: Optional[torch.Tensor], mag: float, positions: torch.Tensor,
+                slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, H: int, G: int, D: int, Dv: int,
+                rot: int) -> torch.Tensor:
+    """Rows [q (H x D) | k (G x D) | v (G x Dv)] -> q [T, H, D] with rotary positions on the first `rot` entries of
+    each head (pairs (i, i + rot/2), angle = position * inv_freq[i] in fp32, cos and sin times `mag`); the rotated
+    keys and the values are appended to the paged cache [NB, G, BS, D] / [NB, G, BS, Dv] at `slots` (-1: skipped)."""
+    if _ref(qkv):
+        return ref.rope_append(qkv, inv_freq, mag, positions, slots, k_cache, v_cache, H, G, D, Dv, rot)
+    lib = require_mixers()
+    T = qkv.shape[0]
+    assert qkv.is_contiguous() and qkv.shape[1] == (H + G) * D + G * Dv and k_cache.dtype == qkv.dtype == v_cache.dtype
+    assert k_cache.shape[1:] == (G, k_cache.shape[2], D) and v_cache.shape == (k_cache.shape[0], G, k_cache.shape[2], Dv)
+    assert positions.dtype == torch.int32 and slots.dtype == torch.int32 and positions.shape[0] >= T and slots.shape[0] >= T
+    assert rot == 0 or (inv_freq.dtype == torch.float32 and inv_freq.numel() * 2 == rot and rot <= D)
+    q = torch.empty((T, H, D), dtype=qkv.dtype, device=qkv.device)
+    check(lib.ka_rope_append(_p(q), _p(qkv), _p(inv_freq), float(mag), _p(positions), _p(slots), _p(k_cache), _p(v_cache),
+                             T, H, G, D, Dv, rot, k_cache.shape[2], _f32(qkv), _stream()), "rope_append")
+    return q
+
+
+SLIDING_TILE = True   # bf16 sliding attention on the matrix cores where the shape allows (False: the vector kernel)
+
+
+def sliding_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                      q_starts: Optional[torch.Tensor], positions: torch.Tensor, slots: torch.Tensor,
+                      gate_src: Optional[torch.Tensor], g_off: int, window: int, keep_first: int, scale: float) -> torch.Tensor:
+    """Softmax attention with grouped keys / values over a paged cache: the query at position p sees the keys
+    j <= p with p - j < window or j < keep_first (window 0: all of 0 .. p; kept keys stay at their own positions).
+    Head h's result is multiplied by sigmoid(gate_src[t, g_off + h]) (gate_src None: no gate).
+    q [T, H, D] -> [T, H * Dv].  q_starts None: row t is block-table row t (a decode step)."""
+    if _ref(q):
+        return ref.sliding_attention(q, k_cache, v_cache, block_tables, q_starts, positions, slots, gate_src, g_off,
+                                     window, keep_first, scale)
+    lib = require_mixers()
+    T, H, D = q.shape
+    G, BS, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    assert q.is_contiguous() and k_cache.dtype == q.dtype == v_cache.dtype and k_cache.shape[3] == D and H % G == 0
+    assert block_tables.dtype == torch.int32 and block_tables.is_contiguous() and block_tables.dim() == 2
+    assert positions.dtype == torch.int32 and slots.dtype == torch.int32 and positions.shape[0] >= T and slots.shape[0] >= T
+    assert q_starts is None or (q_starts.dtype == torch.int32 and q_starts.shape[0] == block_tables.shape[0] + 1)
+    assert q_starts is not None or block_tables.shape[0] >= T
+    gs = 0
+    if gate_src is not None:
+        assert gate_src.dtype == q.dtype and gate_src.is_contiguous() and gate_src.shape[0] >= T
+        gs = gate_src.shape[1]
+        assert 0 <= g_off and g_off + H <= gs
+    out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
+    check(lib.ka_sliding_attention(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(q_starts),
+                                   block_tables.shape[0], _p(positions), _p(slots), _p(gate_src), gs, g_off, T, H, G, D, Dv,
+                                   int(window), int(keep_first), BS, block_tables.shape[1], float(scale), _f32(q),
+                                   0 if SLIDING_TILE else 1, _stream()), "sliding_attention")
+    return out
+
+
+def delta_prep(cv: torch.Tensor, beta_src: torch.Tensor, b_off: int, a_src: torch.Tensor, a_off: int, A_log: torch.Tensor,
+               dt_bias: torch.Tensor, H: int, G: int, D: int, channel: bool):
+    """The fp32 inputs of the delta rule from the convolved rows cv = [q (G x D) | k (G x D) | ...]:
+    qk [T, 2, G, D]: q and k as unit vectors per head, x / sqrt(sum x^2 + 1e-6), q also times D^-1/2;
+    beta [T, H] = sigmoid(beta_src[:, b_off : b_off + H]);
+    decay = exp(-exp(A_log[h]) * softplus(a + dt_bias)): [T, H] from a = a_src[:, a_off : a_off + H], or, channel,
+    [T, H, D] from H * D columns (one decay per head and key channel)."""
+    if _ref(cv):
+        return ref.delta_prep(cv, beta_src, b_off, a_src, a_off, A_log, dt_bias, H, G, D, channel)
+    lib = require_mixers()
+    T = cv.shape[0]
+    n = H * D if channel else H
+    assert cv.is_contiguous() and cv.shape[1] >= 2 * G * D and beta_src.is_contiguous() and a_src.is_contiguous()
+    assert beta_src.dtype == cv.dtype == a_src.dtype and b_off + H <= beta_src.shape[1] and a_off + n <= a_src.shape[1]
+    assert A_log.dtype == torch.float32 and A_log.numel() == H and dt_bias.dtype == torch.float32 and dt_bias.numel() == n
+    qk = torch.empty((T, 2, G, D), dtype=torch.float32, device=cv.device)
+    beta = torch.empty((T, H), dtype=torch.float32, device=cv.device)
+    decay = torch.empty((T, H, D) if channel else (T, H), dtype=torch.float32, device=cv.device)
+    check(lib.ka_delta_prep(_p(qk), _p(beta), _p(decay), _p(cv), cv.shape[1], _p(beta_src), beta_src.shape[1], b_off,
+                            _p(a_src), a_src.shape[1], a_off, _p(A_log), _p(dt_bias), T, H, G, D, int(bool(channel)),
+                            _f32(cv), _stream()), "delta_prep")
+    return qk, beta, decay
+
+
+def delta_scan(qk: torch.Tensor, v_src: torch.Tensor, v_off: int, beta: torch.Tensor, decay: torch.Tensor,
+               st_S: torch.Tensor, seq_slots: torch.Tensor, q_starts: Optional[torch.Tensor], positions: torch.Tensor,
+               H: int, G: int, D: int, Dv: int) -> torch.Tensor:
+    """The gated delta rule over each sequence's rows, from / into the memory of its slot (st_S [slots, H, Dv, D]
+    fp32; a sequence whose first row is at position 0 starts from zero, so slots are reused without clearing).
+    Per head, with q, k = qk[t, 0 / 1, h // (H / G)], v = v_src[t, v_off + h * Dv ...]:
+      S <- decay * S  (decay [T, H]: the whole memory; [T, H, D]: the rows of each key channel)
+      u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
+    q_starts None: row t is sequence t.  -> [T, H * Dv] fp32."""
+    if _ref(qk):
+        return ref.delta_scan(qk, v_src, v_off, beta, decay, st_S, seq_slots, q_starts, positions, H, G, D, Dv)
+    lib = require_mixers()
+    T = qk.shape[0]
+    nseq = seq_slots.shape[0]
+    channel = decay.dim() == 3
+    assert qk.dtype == torch.float32 and qk.shape == (T, 2, G, D) and qk.is_contiguous() and H % G == 0
+    assert v_src.is_contiguous() and v_off + H * Dv <= v_src.shape[1] and v_src.shape[0] >= T
+    assert beta.dtype == decay.dtype == torch.float32 and beta.shape == (T, H) and beta.is_contiguous()
+    assert decay.is_contiguous() and decay.shape == ((T, H, D) if channel else (T, H))
+    assert st_S.dtype == torch.float32 and st_S.shape[1:] == (H, Dv, D) and st_S.is_contiguous()
+    assert seq_slots.dtype == torch.int32 and positions.dtype == torch.int32 and positions.shape[0] >= T
+    assert (q_starts is None and nseq <= T) or (q_starts is not None and q_starts.dtype == torch.int32
+                                                 and q_starts.shape[0] == nseq + 1)
+    out = torch.zeros((T, H * Dv), dtype=torch.float32, device=qk.device)
+    check(lib.ka_delta_scan(_p(out), _p(qk), _p(v_src), v_src.shape[1], v_off, _p(beta), _p(decay), _p(st_S),
+                            _p(seq_slots), _p(q_starts), nseq, _p(positions), H, G, D, Dv, int(channel), _f32(v_src),
+                            _stream()), "delta_scan")
     return out

@@ -320,15 +320,16 @@ def mlstm_scan(proj, q_off: int, k_off: int, v_off: int, gates, st_S, st_n, st_m
     return out, dens
 
 
-def headnorm_gate(o, proj, g_off: int, w, H: int, Dv: int, eps: float, out_dtype, den=None) -> torch.Tensor:
+def headnorm_gate(o, proj, g_off: int, w, H: int, Dv: int, eps: float, out_dtype, den=None, silu: bool = False) -> torch.Tensor:
     """Each head of o (divided by den [T, H] first, if given) divided by its root mean square, times w, times
-    sigmoid(gate columns of proj)."""
+    sigmoid(gate columns of proj) (silu: times silu of them)."""
     T = o.shape[0]
     oh = o.view(T, H, Dv)
     if den is not None:
         oh = oh / den[:, :, None]
     y = (oh / torch.sqrt((oh * oh).mean(-1, keepdim=True) + eps)).reshape(T, H * Dv) * w.float()
-    return (y * torch.sigmoid(proj[:, g_off:g_off + H * Dv].float())).to(out_dtype)
+    g = proj[:, g_off:g_off + H * Dv].float()
+    return (y * (F.silu(g) if silu else torch.sigmoid(g))).to(out_dtype)
 
 
 def _rot(x, positions, inv_freq, dims: int):
@@ -420,4 +421,164 @@ def moe_experts(h, w_gu, w_down, ids, w) -> torch.Tensor:
         tok, slot = torch.nonzero(ids == e, as_tuple=True)
         y = F.linear(silu_mul(F.linear(h[tok], w_gu[e])), w_down[e])
         out.index_add_(0, tok, y.float() * w[tok, slot][:, None])
+    return out
+
+
+# ------------------------------------------------------------------------------------------------
+# Dynamic-Tanh norm, scaled residual sums, short convolutions over state slots, rotary positions with a
+# frequency table, sliding-window attention that keeps the first tokens, the gated delta rule
+# (models/suvapel.py): the ops of ops/mixers.py on CPU tensors, fp32 wherever the kernels are.
+def dyt_norm(x, alpha, w, b, out_dtype):
+    """tanh(alpha * x) * w + b (alpha: a one-element tensor)."""
+    return (torch.tanh(alpha.float() * x.float()) * w.float() + b.float()).to(out_dtype)
+
+
+def residual_mix(x, ys, coefs, out_dtype, want_copy: bool, dyt):
+    """x += sum_i coefs[i] * ys[i] in place (fp32); -> (x in out_dtype if want_copy, dyt_norm(x, *dyt) if dyt)."""
+    acc = None
+    for y, c in zip(ys, coefs):
+        acc = y.float() * c if acc is None else acc + y.float() * c
+    x += acc
+    return (x.to(out_dtype) if want_copy else None), (dyt_norm(x, *dyt, out_dtype) if dyt is not None else None)
+
+
+def rms_residual(x, y, w, mult: float, eps: float, out_dtype, dyt):
+    """x += mult * y / sqrt(mean(y^2) + eps) * w in place; -> dyt_norm(x, *dyt) if dyt."""
+    yf = y.float()
+    x += mult * (yf / torch.sqrt((yf * yf).mean(-1, keepdim=True) + eps) * w.float())
+    return dyt_norm(x, *dyt, out_dtype) if dyt is not None else None
+
+
+def gelu_gate_embed(z, table, ids, col0: int):
+    """gelu_tanh(z) * table[ids, col0 : col0 + z.shape[1]]."""
+    e = table[ids.long().clamp(0, table.shape[0] - 1), col0:col0 + z.shape[1]].float()
+    return (F.gelu(z.float(), approximate="tanh") * e).to(z.dtype)
+
+
+def silu_mul_bias(proj, off: int, ff: int, bias):
+    """silu(proj[:, off : off + ff] + bias[:ff]) * (proj[:, off + ff : off + 2 ff] + bias[ff:])."""
+    g = proj[:, off:off + ff].float() + bias[:ff].float()
+    u = proj[:, off + ff:off + 2 * ff].float() + bias[ff:].float()
+    return (F.silu(g) * u).to(proj.dtype)
+
+
+def short_conv(proj, off: int, C: int, w, state, seq_slots, q_starts, positions, act: bool):
+    """y_t = sum_j w[:, j] * u_(t - taps + 1 + j) per channel over each sequence's rows, u = proj[:, off : off + C];
+    inputs before this step come from state[slot] [taps - 1, C] (the sequence's last inputs, newest last), inputs
+    before position 0 are zero; the state is then advanced by the step's rows.  act: silu on the result."""
+    T = proj.shape[0]
+    taps = w.shape[1]
+    out = torch.zeros((T, C), dtype=proj.dtype, device=proj.device)
+    slots, pos = seq_slots.tolist(), positions.tolist()
+    for i, a, b in _seq_of(T, q_starts):
+        sl = slots[i] if i < len(slots) else -1
+        if sl < 0 or b <= a:
+            continue
+        u = proj[a:b, off:off + C].float()
+        hist = state[sl].float() if taps > 1 else u[:0]
+        if pos[a] < taps - 1 and taps > 1:   # what lies before position 0 is zero
+            hist = hist.clone()
+            hist[:taps - 1 - pos[a]] = 0.0
+        full = torch.cat([hist, u])                                   # row r of the step is full[r + taps - 1]
+        y = sum(w[:, j].float() * full[j:j + (b - a)] for j in range(taps))
+        out[a:b] = (F.silu(y) if act else y).to(proj.dtype)
+        if taps > 1:
+            state[sl] = full[-(taps - 1):].to(state.dtype)
+    return out
+
+
+def rope_append(qkv, inv_freq, mag: float, positions, slots, k_cache, v_cache, H: int, G: int, D: int, Dv: int, rot: int):
+    """Rows [q (H x D) | k (G x D) | v (G x Dv)]: rotary positions (angle = position * inv_freq, cos and sin times
+    mag) on the first `rot` entries of every q and k head; -> q [T, H, D]; k and v go to the paged cache
+    [NB, G, BS, D] / [NB, G, BS, Dv] at `slots`."""
+    T = qkv.shape[0]
+    q = qkv[:, :H * D].float().view(T, H, D)
+    k = qkv[:, H * D:(H + G) * D].float().view(T, G, D)
+    v = qkv[:, (H + G) * D:(H + G) * D + G * Dv].view(T, G, Dv)
+    half = rot // 2
+    if half:
+        ang = positions[:T].float()[:, None] * inv_freq.float()[None, :]
+        c, s = (torch.cos(ang) * mag)[:, None, :], (torch.sin(ang) * mag)[:, None, :]
+
+        def turn(x):
+            a, b = x[..., :half], x[..., half:rot]
+            return torch.cat([a * c - b * s, b * c + a * s, x[..., rot:]], dim=-1)
+
+        q, k = turn(q), turn(k)
+    sl = slots[:T].long()
+    ok = sl >= 0
+    if ok.any():
+        bs = k_cache.shape[2]
+        k_cache[sl[ok] // bs, :, sl[ok] % bs] = k[ok].to(k_cache.dtype)
+        v_cache[sl[ok] // bs, :, sl[ok] % bs] = v[ok].to(v_cache.dtype)
+    return q.to(qkv.dtype).contiguous()
+
+
+def sliding_attention(q, k_cache, v_cache, block_tables, q_starts, positions, slots, gate_src, g_off: int, window: int,
+                      keep_first: int, scale: float):
+    """q [T, H, D] -> [T, H * Dv]: softmax attention over the keys j <= p with p - j < window or j < keep_first
+    (window 0: all); head h's result times sigmoid(gate_src[t, g_off + h]) (gate_src None: no gate)."""
+    T, H, D = q.shape
+    G, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    rep = H // G
+    out = torch.zeros(T, H * Dv, dtype=q.dtype, device=q.device)
+    pos_l, slot_l = positions.tolist(), slots.tolist()
+    for i, a, b in _seq_of(T, q_starts):
+        for t in range(a, b):
+            if slot_l[t] < 0:
+                continue
+            p = pos_l[t]
+            lo = max(0, p - window + 1) if window > 0 else 0
+            js = torch.cat([torch.arange(0, min(keep_first, lo)), torch.arange(lo, p + 1)])
+            pages = block_tables[i].long()[js // bs]
+            k = k_cache[pages, :, js % bs, :].float().repeat_interleave(rep, dim=1)   # [n, H, D]
+            v = v_cache[pages, :, js % bs, :].float().repeat_interleave(rep, dim=1)
+            w = torch.softmax(torch.einsum("hd,nhd->hn", q[t].float(), k) * scale, dim=1)
+            o = torch.einsum("hn,nhd->hd", w, v)
+            if gate_src is not None:
+                o = o * torch.sigmoid(gate_src[t, g_off:g_off + H].float())[:, None]
+            out[t] = o.reshape(-1).to(q.dtype)
+    return out
+
+
+def delta_prep(cv, beta_src, b_off: int, a_src, a_off: int, A_log, dt_bias, H: int, G: int, D: int, channel: bool):
+    """From the convolved rows cv = [q (G x D) | k (G x D) | ...]: unit q (times D^-1/2) and unit k per head
+    (x / sqrt(sum x^2 + 1e-6)) -> qk [T, 2, G, D]; beta = sigmoid(beta_src[:, b_off : b_off + H]) [T, H]; decay =
+    exp(-exp(A_log) * softplus(a + dt_bias)) [T, H] (a = a_src[:, a_off : a_off + H]) or, channel, [T, H, D] (a of
+    H * D columns).  All fp32."""
+    T = cv.shape[0]
+    x = cv[:, :2 * G * D].float().view(T, 2, G, D)
+    x = x / torch.sqrt((x * x).sum(-1, keepdim=True) + 1e-6)
+    x[:, 0] *= D ** -0.5
+    beta = torch.sigmoid(beta_src[:, b_off:b_off + H].float())
+    n = H * D if channel else H
+    sp = F.softplus(a_src[:, a_off:a_off + n].float() + dt_bias.float())
+    rate = torch.exp(A_log.float())
+    decay = torch.exp(-(rate[None, :, None] * sp.view(T, H, D))) if channel else torch.exp(-(rate[None, :] * sp))
+    return x.contiguous(), beta.contiguous(), decay.contiguous()
+
+
+def delta_scan(qk, v_src, v_off: int, beta, decay, st_S, seq_slots, q_starts, positions, H: int, G: int, D: int, Dv: int):
+    """The gated delta rule over each sequence's rows, from / into st_S[slot] [H, Dv, D] (zero when the first row's
+    position is 0): S <- decay * S (per head or per key channel); u = beta (v - S^T k); S <- S + k u^T; o = S^T q.
+    -> [T, H * Dv] fp32."""
+    T = qk.shape[0]
+    rep = H // G
+    out = torch.zeros((T, H * Dv), dtype=torch.float32, device=qk.device)
+    slots, pos = seq_slots.tolist(), positions.tolist()
+    for i, a, b in _seq_of(T, q_starts):
+        sl = slots[i] if i < len(slots) else -1
+        if sl < 0 or b <= a:
+            continue
+        S = torch.zeros(H, Dv, D) if pos[a] == 0 else st_S[sl].clone()
+        for t in range(a, b):
+            q = qk[t, 0].repeat_interleave(rep, dim=0)      # [H, D]
+            k = qk[t, 1].repeat_interleave(rep, dim=0)
+            v = v_src[t, v_off:v_off + H * Dv].float().view(H, Dv)
+            g = decay[t].view(H, 1, -1)                     # [H, 1, 1 or D]
+            S = S * g
+            u = beta[t][:, None] * (v - torch.einsum("hvd,hd->hv", S, k))
+            S = S + u[:, :, None] * k[:, None, :]
+            out[t] = torch.einsum("hvd,hd->hv", S, q).reshape(-1)
+        st_S[sl] = S
     return out
