@@ -1,0 +1,238 @@
+// KA_HIP_LIB: mixers
+// KA_HIPCC_FLAGS: -Xclang -target-feature -Xclang -packed-fp32-ops
+// Softmax attention with grouped keys / values over a paged cache, with a sliding window that also keeps the
+// sequence's first tokens (models/suvapel.py):
+//
+//   visible(p, j) = j <= p and (p - j < window or j < keep_first)      (window 0: every j <= p)
+//   a kept key is rotated and masked by the position it was written at, like any other key;
+//   head h's result is multiplied by sigmoid(gate[t, h]), one number per token and head (gate null: none).
+//
+// `rope_append`: rows [q (H x D) | k (G x D) | v (G x Dv)] -> q [T, H, D], rotary positions on the first `rot`
+// entries of every q and k head (pairs (i, i + rot/2), angle = position * inv_freq[i] in fp32, cos and sin times
+// `mag`: a frequency table and a magnitude are what YaRN-style scalings come down to); the rotated keys and the
+// values go to the paged cache.  Cache layout: k_cache [NB, G, BS, D], v_cache [NB, G, BS, Dv], token-major pages;
+// slot = page * BS + offset (-1: a padding row, nothing is written or attended).
+//
+// `sliding_attention`, vector kernel: one workgroup per (token, key/value head) with the H / G query heads that
+// share it.  The visible keys (the kept first ones, then the window) are walked in tiles of 64 with an online
+// softmax: scores by one thread per (query head, key), the tile's maximum / sum per head by one wave, weights x
+// values by one thread per output entry.  Scores, weights and all sums are fp32; AT (bf16_t or float) is the type
+// of q, the cache, the gate and the output.  A decode step is the same launch with one token per sequence, so a
+// position's result does not depend on whether it was a prompt row or a decoded one.
+#include "rows_f32.h"
+
+namespace {
+using namespace rows;
+
+constexpr int KT = 64;        // keys per tile
+constexpr int MAX_REP = 16;   // query heads per key/value head
+constexpr int MAX_ACC = 8;    // output entries per thread: (H / G) * Dv <= NT * MAX_ACC
+
+template <typename AT>
+__global__ __launch_bounds__(NT) void rope_append_kernel(AT* __restrict__ q_out, const AT* __restrict__ qkv,
+                                                         const float* __restrict__ inv_freq, float mag,
+                                                         const int* __restrict__ positions, const int* __restrict__ slots,
+                                                         AT* __restrict__ k_cache, AT* __restrict__ v_cache, int H, int G,
+                                                         int D, int Dv, int rot, int BS) {
+  const int t = blockIdx.x;
+  const int half = rot >> 1;
+  const float pos = (float)positions[t];
+  const int slot = slots[t];
+  const AT* row = qkv + (size_t)t * ((H + G) * D + G * Dv);
+  const size_t page = slot >= 0 ? (size_t)(slot / BS) : 0, offs = slot >= 0 ? (size_t)(slot % BS) : 0;
+  for (int idx = threadIdx.x; idx < (H + G) * D; idx += NT) {
+    const int hh = idx / D, i = idx % D;
+    if (hh >= H && slot < 0) break;
+    float o = ldf(row + idx);
+    if (i < rot) {
+      const int j = i < half ? i : i - half;
+      const float partner = ldf(row + (i < half ? idx + half : idx - half));
+      float sn, cs;
+      sincosf(pos * inv_freq[j], &sn, &cs);
+      sn *= mag;
+      cs *= mag;
+      o = i < half ? o * cs - partner * sn : o * cs + partner * sn;
+    }
+    if (hh < H) stf(q_out + (size_t)t * H * D + idx, o);
+    else stf(k_cache + ((page * G + (hh - H)) * BS + offs) * D + i, o);
+  }
+  if (slot < 0) return;
+  const AT* vrow = row + (H + G) * D;
+  for (int idx = threadIdx.x; idx < G * Dv; idx += NT)
+    v_cache[((page * G + idx / Dv) * BS + offs) * Dv + idx % Dv] = vrow[idx];
+}
+
+struct SlideArgs {
+  const int* block_tables;   // [num_seqs, max_blocks]
+  const int* q_starts;       // [num_seqs + 1] or null (token t is block-table row t)
+  const int* positions;      // [T]
+  const int* slots;          // [T]
+  int num_seqs, H, G, D, Dv, window, keep_first, BS, max_blocks;
+  int gs, g_off;             // gate row stride and column offset
+  float scale;
+};
+
+template <typename AT>
+__global__ __launch_bounds__(NT) void sliding_attention_kernel(AT* __restrict__ out, const AT* __restrict__ q,
+                                                               const AT* __restrict__ k_cache,
+                                                               const AT* __restrict__ v_cache, const AT* __restrict__ gate,
+                                                               SlideArgs a) {
+  extern __shared__ float lds[];
+  const int H = a.H, G = a.G, D = a.D, Dv = a.Dv, BS = a.BS;
+  const int rep = H / G;
+  float* qs = lds;                  // [rep * D]
+  float* sc = qs + rep * D;         // [rep * KT] scores, then weights of the tile
+  __shared__ float s_m[MAX_REP], s_l[MAX_REP], s_c[MAX_REP];   // running maximum, running sum, the tile's rescale
+  __shared__ int s_row[KT];         // cache row (page * G + g) * BS + offset of each key of the tile
+  const int t = blockIdx.x, g = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int RV = rep * Dv;
+  AT* orow = out + (size_t)t * H * Dv + (size_t)g * RV;
+  if (a.slots[t] < 0 || (a.q_starts != nullptr && t >= a.q_starts[a.num_seqs])) {
+    for (int i = threadIdx.x; i < RV; i += NT) stf(orow + i, 0.f);
+    return;
+  }
+  const int p = a.positions[t];
+  const int seq = seq_of(a.q_starts, a.num_seqs, t);
+  const int* bt = a.block_tables + (size_t)seq * a.max_blocks;
+  const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;   // first position of the window
+  const int nk0 = min(a.keep_first, lo);                        // kept first positions that lie before the window
+  const int n = nk0 + (p - lo + 1);
+  for (int i = threadIdx.x; i < rep * D; i += NT) qs[i] = ldf(q + ((size_t)t * H + (size_t)g * rep) * D + i);
+  if (threadIdx.x < rep) {
+    s_m[threadIdx.x] = -INFINITY;
+    s_l[threadIdx.x] = 0.f;
+  }
+  float acc[MAX_ACC];
+#pragma unroll
+  for (int u = 0; u < MAX_ACC; ++u) acc[u] = 0.f;
+  for (int k0 = 0; k0 < n; k0 += KT) {
+    const int nk = min(KT, n - k0);
+    __syncthreads();
+    if (threadIdx.x < nk) {
+      const int i = k0 + threadIdx.x;
+      const int pos = i < nk0 ? i : lo + (i - nk0);
+      s_row[threadIdx.x] = (bt[pos / BS] * G + g) * BS + pos % BS;
+    }
+    __syncthreads();
+    for (int it = threadIdx.x; it < rep * KT; it += NT) {
+      const int r = it / KT, j = it % KT;
+      float s = -INFINITY;
+      if (j < nk) {
+        const AT* kr = k_cache + (size_t)s_row[j] * D;
+        const float* qg = qs + r * D;
+        s = 0.f;
+        if constexpr (sizeof(AT) == 2) {
+          if ((D & 7) == 0) {   // 16-byte loads: 8 bf16 key entries against 8 fp32 query entries from LDS
+            for (int i = 0; i < D; i += 8) {
+              const uint4 kv = *reinterpret_cast<const uint4*>(kr + i);
+              const f32x4 qa = *reinterpret_cast<const f32x4*>(qg + i), qb = *reinterpret_cast<const f32x4*>(qg + i + 4);
+              s += qa[0] * lo_f(kv.x) + qa[1] * hi_f(kv.x) + qa[2] * lo_f(kv.y) + qa[3] * hi_f(kv.y) +
+                   qb[0] * lo_f(kv.z) + qb[1] * hi_f(kv.z) + qb[2] * lo_f(kv.w) + qb[3] * hi_f(kv.w);
+            }
+          } else {
+            for (int i = 0; i < D; ++i) s += qg[i] * ldf(kr + i);
+          }
+        } else {
+          if ((D & 3) == 0) {
+            for (int i = 0; i < D; i += 4) {
+              const f32x4 kv = *reinterpret_cast<const f32x4*>(kr + i);
+              const f32x4 qa = *reinterpret_cast<const f32x4*>(qg + i);
+              s += qa[0] * kv[0] + qa[1] * kv[1] + qa[2] * kv[2] + qa[3] * kv[3];
+            }
+          } else {
+            for (int i = 0; i < D; ++i) s += qg[i] * ldf(kr + i);
+          }
+        }
+        s *= a.scale;
+      }
+      sc[it] = s;
+    }
+    __syncthreads();
+    for (int r = wave; r < rep; r += NW) {      // the tile's place in head r's running softmax
+      const float s = sc[r * KT + lane];
+      const float mo = s_m[r];
+      const float m = fmaxf(mo, wave_max(s));   // finite: a tile holds at least one key
+      const float e = s == -INFINITY ? 0.f : expf(s - m);
+      const float sum = wave_sum(e);
+      sc[r * KT + lane] = e;
+      if (lane == 0) {
+        const float corr = mo == -INFINITY ? 0.f : expf(mo - m);
+        s_c[r] = corr;
+        s_l[r] = s_l[r] * corr + sum;
+        s_m[r] = m;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < MAX_ACC; ++u) {
+      const int i = threadIdx.x + u * NT;
+      if (i < RV) {
+        const int r = i / Dv, d = i % Dv;
+        const float* wr = sc + r * KT;
+        float s = acc[u] * s_c[r];
+        for (int j = 0; j < nk; ++j) s += wr[j] * ldf(v_cache + (size_t)s_row[j] * Dv + d);
+        acc[u] = s;
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < MAX_ACC; ++u) {
+    const int i = threadIdx.x + u * NT;
+    if (i < RV) {
+      const int r = i / Dv;
+      float o = acc[u] / s_l[r];
+      if (gate != nullptr) o *= 1.0f / (1.0f + expf(-ldf(gate + (size_t)t * a.gs + a.g_off + g * rep + r)));
+      stf(orow + i, o);
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int ka_rope_append(void* q_out, const void* qkv, const float* inv_freq, float mag, const int* positions,
+                              const int* slots, void* k_cache, void* v_cache, int T, int H, int G, int D, int Dv, int rot,
+                              int BS, int f32, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (D <= 0 || Dv <= 0 || rot < 0 || rot > D || (rot & 1) || BS <= 0 || H <= 0 || G <= 0 || (rot > 0 && inv_freq == nullptr))
+    return (int)hipErrorInvalidValue;
+  if (f32)
+    rope_append_kernel<float><<<T, NT, 0, st>>>((float*)q_out, (const float*)qkv, inv_freq, mag, positions, slots,
+                                                (float*)k_cache, (float*)v_cache, H, G, D, Dv, rot, BS);
+  else
+    rope_append_kernel<bf16_t><<<T, NT, 0, st>>>((bf16_t*)q_out, (const bf16_t*)qkv, inv_freq, mag, positions, slots,
+                                                 (bf16_t*)k_cache, (bf16_t*)v_cache, H, G, D, Dv, rot, BS);
+  KA_CHECK_LAUNCH();
+}
+
+// mode 0: the fastest kernel the shape allows; 1: the vector kernel
+extern "C" int ka_sliding_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                    const int* block_tables, const int* q_starts, int num_seqs, const int* positions,
+                                    const int* slots, const void* gate, int gs, int g_off, int T, int H, int G, int D,
+                                    int Dv, int window, int keep_first, int BS, int max_blocks, float scale, int f32,
+                                    int mode, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (H <= 0 || G <= 0 || H % G || H / G > MAX_REP || (H / G) * Dv > NT * MAX_ACC || D <= 0 || Dv <= 0 || BS <= 0 ||
+      window < 0 || keep_first < 0 || num_seqs <= 0)
+    return (int)hipErrorInvalidValue;
+  (void)mode;
+  const int rep = H / G;
+  const size_t lds = (size_t)(rep * D + rep * KT) * sizeof(float);
+  if (lds > 60 * 1024) return (int)hipErrorInvalidValue;
+  SlideArgs a{block_tables, q_starts, positions, slots, num_seqs, H, G, D, Dv, window, keep_first, BS, max_blocks, gs, g_off, scale};
+  if (lds > 48 * 1024) {
+    const void* fn = f32 ? reinterpret_cast<const void*>(sliding_attention_kernel<float>)
+                         : reinterpret_cast<const void*>(sliding_attention_kernel<bf16_t>);
+    const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+  }
+  const dim3 grid(T, G);
+  if (f32)
+    sliding_attention_kernel<float><<<grid, NT, lds, st>>>((float*)out, (const float*)q, (const float*)k_cache,
+                                                           (const float*)v_cache, (const float*)gate, a);
+  else
+    sliding_attention_kernel<bf16_t><<<grid, NT, lds, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache,
+                                                            (const bf16_t*)v_cache, (const bf16_t*)gate, a);
+  KA_CHECK_LAUNCH();
+}

@@ -129,12 +129,13 @@ __global__ __launch_bounds__(NT) void silu_mul_rows_kernel(AT* __restrict__ out,
 }
 
 // one wave per head: o [T, H * Dv] fp32 -> out in AT; the gate columns sit in `proj` rows of stride ps at g_off
+// (sigmoid of them, or silu of them)
 // den [T, H] (optional): the head's entries are first divided by den[t, h]
 template <typename AT>
 __global__ __launch_bounds__(NT) void headnorm_gate_kernel(AT* __restrict__ out, const float* __restrict__ o,
                                                            const float* __restrict__ den, const AT* __restrict__ proj,
                                                            int ps, int g_off, const float* __restrict__ w, int H, int Dv,
-                                                           float eps) {
+                                                           float eps, int silu) {
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int h = wave; h < H; h += NW) {
     const float* oh = o + ((size_t)t * H + h) * Dv;
@@ -147,7 +148,7 @@ __global__ __launch_bounds__(NT) void headnorm_gate_kernel(AT* __restrict__ out,
     const float inv = rd / sqrtf(wave_sum(ss) / (float)Dv + eps);
     for (int i = lane; i < Dv; i += 64) {
       const float g = ldf(proj + (size_t)t * ps + g_off + h * Dv + i);
-      stf(out + ((size_t)t * H + h) * Dv + i, oh[i] * inv * w[h * Dv + i] / (1.f + expf(-g)));
+      stf(out + ((size_t)t * H + h) * Dv + i, oh[i] * inv * w[h * Dv + i] * (silu ? g : 1.f) / (1.f + expf(-g)));
     }
   }
 }
@@ -204,10 +205,11 @@ extern "C" int ka_silu_mul_rows(void* out, const void* gu, int rows_, int ff, in
   KA_CHECK_LAUNCH();
 }
 
+// silu: the gate is silu(g) = g * sigmoid(g) instead of sigmoid(g)
 extern "C" int ka_headnorm_gate(void* out, const float* o, const float* den, const void* proj, int ps, int g_off,
-                                const float* w, int T, int H, int Dv, float eps, int f32, hipStream_t st) {
+                                const float* w, int T, int H, int Dv, float eps, int silu, int f32, hipStream_t st) {
   if (T <= 0) return 0;
-  if (f32) headnorm_gate_kernel<float><<<T, NT, 0, st>>>((float*)out, o, den, (const float*)proj, ps, g_off, w, H, Dv, eps);
-  else headnorm_gate_kernel<bf16_t><<<T, NT, 0, st>>>((bf16_t*)out, o, den, (const bf16_t*)proj, ps, g_off, w, H, Dv, eps);
+  if (f32) headnorm_gate_kernel<float><<<T, NT, 0, st>>>((float*)out, o, den, (const float*)proj, ps, g_off, w, H, Dv, eps, silu);
+  else headnorm_gate_kernel<bf16_t><<<T, NT, 0, st>>>((bf16_t*)out, o, den, (const bf16_t*)proj, ps, g_off, w, H, Dv, eps, silu);
   KA_CHECK_LAUNCH();
 }
