@@ -236,3 +236,109 @@ def load_checkpoint(path: str):
             raise ValueError(e["dtype"])
         T[name] = a.astype(np.float64).reshape(e["shape"])
     return cfg, T
+
+
+# ---- small configurations and random checkpoints for the tests -----------------------------------------
+def delta_mixer_cfg(heads=2, kv_heads=1, dim=8, vdim=12, conv=4):
+    return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv}
+
+
+def attention_cfg(heads=4, kv_heads=2, dim=16, vdim=8, conv=2, window=8, keep_first=2, rot_dims=8, base=50000.0,
+                  scaling=(4.0, 64, 8.0, 2.0), scale=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv,
+         "scale": scale if scale is not None else dim ** -0.5}
+    if window:
+        m["mask"] = {"size": window, "keep_first": keep_first}
+    if rot_dims:
+        m["rot"] = {"base": base, "dims": rot_dims}
+        if scaling:
+            m["rot"]["scaling"] = dict(zip(("factor", "original", "fast", "slow"), scaling))
+    return m
+
+
+def delta_layer(ff=24, **kw):
+    return {"type": "delta", "mixer": delta_mixer_cfg(**kw), "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def parallel_layer(left=None, right=None, left_scale=0.75, right_scale=1.1, ff=24):
+    return {"type": "parallel", "mixer": {"left": left or attention_cfg(), "right": right or delta_mixer_cfg(conv=3),
+                                          "left_scale": left_scale, "right_scale": right_scale},
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def make_config(layers, width=32, vocab=96, side=6, mult=0.8, eps=1e-6):
+    c = {"architecture": "Suvapel", "vocab": vocab, "width": width, "norm": {"eps": eps}, "residual_mult": mult,
+         "layers": layers}
+    if side:
+        c["token_side"] = {"dim": side}
+    return c
+
+
+def random_tensors(cfg, seed=0, rank=5):
+    """Random checkpoint tensors for `cfg` as torch bf16 tensors (what a checkpoint stores)."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    h, V = cfg["width"], cfg["vocab"]
+    bf = torch.bfloat16
+
+    def mat(o, i, std=None):
+        return (torch.randn(o, i, generator=g) * (std if std is not None else i ** -0.5)).to(bf)
+
+    def vec(n, lo=0.7, hi=1.3):
+        return (lo + (hi - lo) * torch.rand(n, generator=g)).to(bf)
+
+    def norm(name):
+        return {name: vec(h), name + ".b": (torch.randn(h, generator=g) * 0.1).to(bf),
+                name + ".alpha": (0.3 + 0.5 * torch.rand((), generator=g)).to(bf)}
+
+    def conv(c, taps):
+        return (torch.randn(c, taps, generator=g) * 0.5 + torch.eye(taps)[-1] * 0.8).to(bf)
+
+    def delta(p, m, channel):
+        H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        T = {}
+        for k, n in (("q", G * D), ("k", G * D), ("v", H * Dv)):
+            T[p + k], T[p + k + ".conv"] = mat(n, h, 2.0 * h ** -0.5), conv(n, m["conv"])
+        T[p + "b"] = mat(H, h, 2.0 * h ** -0.5)
+        T[p + "A_log"] = torch.log(0.3 + 4.0 * torch.rand(H, generator=g)).to(bf)
+        T[p + "norm"], T[p + "o"] = vec(Dv), mat(h, H * Dv)
+        if channel:
+            T[p + "a1"], T[p + "a2"] = mat(rank, h), mat(H * D, rank, 2.0 * rank ** -0.5)
+            T[p + "g1"], T[p + "g2"] = mat(rank + 2, h), mat(H * Dv, rank + 2, 2.0 * rank ** -0.5)
+            T[p + "dt_bias"] = (torch.randn(H * D, generator=g) - 2.0).to(bf)
+        else:
+            T[p + "a"], T[p + "g"] = mat(H, h, 2.0 * h ** -0.5), mat(H * Dv, h)
+            T[p + "dt_bias"] = (torch.randn(H, generator=g) - 2.0).to(bf)
+        return T
+
+    T = {"embed": mat(V, h, 1.0), "head": mat(V, h), **norm("final.norm")}
+    side = (cfg.get("token_side") or {}).get("dim", 0)
+    if side:
+        T["side.embed"] = mat(V, side * len(cfg["layers"]), 1.0)
+    for i, L in enumerate(cfg["layers"]):
+        c, m = f"l{i}.", L["mixer"]
+        T.update(norm(c + "norm1"))
+        if L["type"] == "delta":
+            T.update(delta(c + "mix.", m, False))
+        else:
+            a = m["left"]
+            for k, n in (("q", a["heads"] * a["dim"]), ("k", a["kv_heads"] * a["dim"]), ("v", a["kv_heads"] * a["vdim"])):
+                T[c + "mix.left." + k] = mat(n, h, 2.0 * h ** -0.5)
+                T[c + "mix.left." + k + ".conv"] = conv(n, a["conv"])
+            T[c + "mix.left.g"], T[c + "mix.left.o"] = mat(a["heads"], h, 2.0 * h ** -0.5), mat(h, a["heads"] * a["vdim"])
+            T.update(delta(c + "mix.right.", m["right"], True))
+        if L.get("mlp") is not None:
+            ff = L["mlp"]["ff"]
+            for k, o_, i_ in (("gate", ff, h), ("up", ff, h), ("down", h, ff)):
+                T[c + "mlp." + k] = mat(o_, i_)
+                T[c + "mlp." + k + ".b"] = (torch.randn(o_, generator=g) * 0.2).to(bf)
+        if side:
+            T[c + "side.gate"], T[c + "side.proj"] = mat(side, h), mat(h, side)
+            T[c + "side.norm"] = vec(h, 0.2, 0.6)
+    return T
+
+
+def as_arrays(T):
+    """torch tensors -> float64 numpy (what `forward` takes)."""
+    return {k: v.double().numpy() for k, v in T.items()}
