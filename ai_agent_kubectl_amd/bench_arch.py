@@ -4,7 +4,10 @@
 with the same width, heads, head size, feed-forward width, vocabulary and depth (random weights), and with
 `--arch-models ...,kafilorn` a Kafilorn of that width and depth (layers cycling mLSTM + dense, latent attention
 + experts, latent attention on the previous layer's cache + dense; latent ranks W/8 and 3W/8, 8 experts of
-width ff/4 with 2 chosen plus a shared one, two residual streams), go through the same engine path (`build_engine`, the scheduler, `ModelRunner.execute`, hipGraph decode):
+width ff/4 with 2 chosen plus a shared one, two residual streams), and with `...,suvapel` a Suvapel of that width and
+depth (layers alternating a delta rule with attention beside a channel-decay delta rule, window = the chunk, four
+taps, a 64-wide token input; its closest existing model is Kafilorn: recurrent state slots + windowed attention +
+fp32 residual), go through the same engine path (`build_engine`, the scheduler, `ModelRunner.execute`, hipGraph decode):
 B prompts of P tokens are prefilled (in steps of the engine's token budget), then N tokens are
 decoded per sequence.  Reported per model: prefill tokens/s (prompt tokens / time in prefill steps)
 and decode tokens/s (B x decode steps / time in decode steps), from the runner's own step timers.
@@ -25,7 +28,7 @@ SIZES = {
 def _configs(size: str, chunk: int):
     import dataclasses
 
-    from .models.config import PRESETS, ModelConfig, kafilorn_uniform, vivepel_uniform
+    from .models.config import PRESETS, ModelConfig, kafilorn_uniform, suvapel_uniform, vivepel_uniform
 
     W, H, G, D, ff, V, L = SIZES[size]
     ll = ModelConfig(f"llama-{size}-{L}l", "llama", L, W, H, G, D, ff, V, 500000.0)
@@ -33,8 +36,9 @@ def _configs(size: str, chunk: int):
     kk = kafilorn_uniform(f"kafilorn-{size}-{L}l", (L + 2) // 3, W, H, V, ff, experts=8, top=2, expert_ff=ff // 4,
                           window=chunk, streams=2, kv_rank=W // 8, q_rank=3 * W // 8, dim=D, rot_dim=D // 2)
     kk = dataclasses.replace(kk, layers=kk.layers[:L])
-    PRESETS[ll.name], PRESETS[vv.name], PRESETS[kk.name] = ll, vv, kk
-    return ll, vv, kk
+    ss = suvapel_uniform(f"suvapel-{size}-{L}l", L, W, H, G, D, ff, V, window=chunk)
+    PRESETS[ll.name], PRESETS[vv.name], PRESETS[kk.name], PRESETS[ss.name] = ll, vv, kk, ss
+    return ll, vv, kk, ss
 
 
 def run_one(model: str, batch: int, prompt: int, new_tokens: int, warmup: int = 1, device: str = "cuda") -> dict:
@@ -80,8 +84,8 @@ def main(sizes=("2k", "8b"), batch: int = 32, prompt: int = 1024, new_tokens: in
          which=("llama", "vivepel")) -> dict:
     rows = []
     for size in sizes:
-        ll, vv, kk = _configs(size, chunk)
-        for cfg in [c for c, n in ((ll, "llama"), (vv, "vivepel"), (kk, "kafilorn")) if n in which]:
+        ll, vv, kk, ss = _configs(size, chunk)
+        for cfg in [c for c, n in ((ll, "llama"), (vv, "vivepel"), (kk, "kafilorn"), (ss, "suvapel")) if n in which]:
             r = run_one(cfg.name, batch, prompt, new_tokens)
             r["size"] = size
             rows.append(r)
@@ -95,4 +99,8 @@ def main(sizes=("2k", "8b"), batch: int = 32, prompt: int = 1024, new_tokens: in
            "chunk": chunk, "rows": rows, "vivepel_over_llama": ratio}
     if kratio:
         out["kafilorn_over_vivepel"] = kratio
+    sratio = {s: {k: round(by[(s, "suvapel")][k] / by[(s, "kafilorn")][k], 3) for k in ("prefill_tok_s", "decode_tok_s")}
+              for s in sizes if (s, "suvapel") in by and (s, "kafilorn") in by}
+    if sratio:
+        out["suvapel_over_kafilorn"] = sratio
     return out
