@@ -10,16 +10,16 @@
 // `rope_append`: rows [q (H x D) | k (G x D) | v (G x Dv)] -> q [T, H, D], rotary positions on the first `rot`
 // entries of every q and k head (pairs (i, i + rot/2), angle = position * inv_freq[i] in fp32, cos and sin times
 // `mag`: a frequency table and a magnitude are what YaRN-style scalings come down to); the rotated keys and the
-// values go to the paged cache.  Cache layout: k_cache [NB, G, BS, D], v_cache [NB, G, BS, Dv], token-major pages;
-// slot = page * BS + offset (-1: a padding row, nothing is written or attended).
+// values go to the paged cache.  Cache layout: k_cache [NB, G, BS, D] (token-major), v_cache [NB, G, Dv, BS] (a page's
+// values of one entry contiguous); slot = page * BS + offset (-1: a padding row, nothing is written or attended).
 //
 // `sliding_attention`, vector kernel: one workgroup per (token, key/value head) with the H / G query heads that
-// share it.  The visible keys (the kept first ones, then the window) are walked in tiles of 64 with an online
-// softmax: scores by one thread per (query head, key), the tile's maximum / sum per head by one wave, weights x
-// values by one thread per output entry.  Scores, weights and all sums are fp32; AT (bf16_t or float) is the type
+// share it.  The visible keys (the kept first ones, then the window) are walked in page-aligned tiles of 64
+// positions with an online softmax: scores by one thread per (query head, key), the tile's maximum / sum per head by
+// one wave, weights x values by one thread per output entry, a page's values in 16-byte pieces.  Scores, weights and all sums are fp32; AT (bf16_t or float) is the type
 // of q, the cache, the gate and the output.  A decode step is the same launch with one token per sequence, so a
 // position's result does not depend on whether it was a prompt row or a decoded one.
-#include "rows_f32.h"
+#include "attention_window.h"
 
 namespace {
 using namespace rows;
@@ -27,6 +27,7 @@ using namespace rows;
 constexpr int KT = 64;        // keys per tile
 constexpr int MAX_REP = 16;   // query heads per key/value head
 constexpr int MAX_ACC = 8;    // output entries per thread: (H / G) * Dv <= NT * MAX_ACC
+constexpr int TILE_MIN_ROWS = 8;   // steps whose longest run of rows is shorter stay on the vector kernel
 
 template <typename AT>
 __global__ __launch_bounds__(NT) void rope_append_kernel(AT* __restrict__ q_out, const AT* __restrict__ qkv,
@@ -59,18 +60,9 @@ __global__ __launch_bounds__(NT) void rope_append_kernel(AT* __restrict__ q_out,
   if (slot < 0) return;
   const AT* vrow = row + (H + G) * D;
   for (int idx = threadIdx.x; idx < G * Dv; idx += NT)
-    v_cache[((page * G + idx / Dv) * BS + offs) * Dv + idx % Dv] = vrow[idx];
+    v_cache[((page * G + idx / Dv) * Dv + idx % Dv) * BS + offs] = vrow[idx];
 }
 
-struct SlideArgs {
-  const int* block_tables;   // [num_seqs, max_blocks]
-  const int* q_starts;       // [num_seqs + 1] or null (token t is block-table row t)
-  const int* positions;      // [T]
-  const int* slots;          // [T]
-  int num_seqs, H, G, D, Dv, window, keep_first, BS, max_blocks;
-  int gs, g_off;             // gate row stride and column offset
-  float scale;
-};
 
 template <typename AT>
 __global__ __launch_bounds__(NT) void sliding_attention_kernel(AT* __restrict__ out, const AT* __restrict__ q,
@@ -83,7 +75,7 @@ __global__ __launch_bounds__(NT) void sliding_attention_kernel(AT* __restrict__ 
   float* qs = lds;                  // [rep * D]
   float* sc = qs + rep * D;         // [rep * KT] scores, then weights of the tile
   __shared__ float s_m[MAX_REP], s_l[MAX_REP], s_c[MAX_REP];   // running maximum, running sum, the tile's rescale
-  __shared__ int s_row[KT];         // cache row (page * G + g) * BS + offset of each key of the tile
+  __shared__ int s_page[KT];        // (page * G + g) of each page of the tile (KT / BS of them)
   const int t = blockIdx.x, g = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int RV = rep * Dv;
@@ -97,7 +89,6 @@ __global__ __launch_bounds__(NT) void sliding_attention_kernel(AT* __restrict__ 
   const int* bt = a.block_tables + (size_t)seq * a.max_blocks;
   const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;   // first position of the window
   const int nk0 = min(a.keep_first, lo);                        // kept first positions that lie before the window
-  const int n = nk0 + (p - lo + 1);
   for (int i = threadIdx.x; i < rep * D; i += NT) qs[i] = ldf(q + ((size_t)t * H + (size_t)g * rep) * D + i);
   if (threadIdx.x < rep) {
     s_m[threadIdx.x] = -INFINITY;
@@ -106,73 +97,90 @@ __global__ __launch_bounds__(NT) void sliding_attention_kernel(AT* __restrict__ 
   float acc[MAX_ACC];
 #pragma unroll
   for (int u = 0; u < MAX_ACC; ++u) acc[u] = 0.f;
-  for (int k0 = 0; k0 < n; k0 += KT) {
-    const int nk = min(KT, n - k0);
-    __syncthreads();
-    if (threadIdx.x < nk) {
-      const int i = k0 + threadIdx.x;
-      const int pos = i < nk0 ? i : lo + (i - nk0);
-      s_row[threadIdx.x] = (bt[pos / BS] * G + g) * BS + pos % BS;
-    }
-    __syncthreads();
-    for (int it = threadIdx.x; it < rep * KT; it += NT) {
-      const int r = it / KT, j = it % KT;
-      float s = -INFINITY;
-      if (j < nk) {
-        const AT* kr = k_cache + (size_t)s_row[j] * D;
-        const float* qg = qs + r * D;
-        s = 0.f;
-        if constexpr (sizeof(AT) == 2) {
-          if ((D & 7) == 0) {   // 16-byte loads: 8 bf16 key entries against 8 fp32 query entries from LDS
-            for (int i = 0; i < D; i += 8) {
-              const uint4 kv = *reinterpret_cast<const uint4*>(kr + i);
-              const f32x4 qa = *reinterpret_cast<const f32x4*>(qg + i), qb = *reinterpret_cast<const f32x4*>(qg + i + 4);
-              s += qa[0] * lo_f(kv.x) + qa[1] * hi_f(kv.x) + qa[2] * lo_f(kv.y) + qa[3] * hi_f(kv.y) +
-                   qb[0] * lo_f(kv.z) + qb[1] * hi_f(kv.z) + qb[2] * lo_f(kv.w) + qb[3] * hi_f(kv.w);
+  // two spans of positions: the kept first ones [0, nk0), then the window [lo, p]; each is walked in tiles of KT
+  // positions that start on a page border, the positions of a tile outside its span are masked
+  for (int span = 0; span < 2; ++span) {
+    const int sa = span == 0 ? 0 : lo, sb = span == 0 ? nk0 : p + 1;
+    for (int pos0 = (sa / BS) * BS; pos0 < sb; pos0 += KT) {
+      __syncthreads();
+      if (threadIdx.x < KT / BS && pos0 + threadIdx.x * BS < sb) s_page[threadIdx.x] = bt[pos0 / BS + threadIdx.x] * G + g;
+      __syncthreads();
+      for (int it = threadIdx.x; it < rep * KT; it += NT) {
+        const int r = it / KT, j = it % KT;
+        const int pos = pos0 + j;
+        float s = -INFINITY;
+        if (pos >= sa && pos < sb) {
+          const AT* kr = k_cache + ((size_t)s_page[j / BS] * BS + j % BS) * D;
+          const float* qg = qs + r * D;
+          s = 0.f;
+          if constexpr (sizeof(AT) == 2) {
+            if ((D & 7) == 0) {   // 16-byte loads: 8 bf16 key entries against 8 fp32 query entries from LDS
+              for (int i = 0; i < D; i += 8) {
+                const uint4 kv = *reinterpret_cast<const uint4*>(kr + i);
+                const f32x4 qa = *reinterpret_cast<const f32x4*>(qg + i), qb = *reinterpret_cast<const f32x4*>(qg + i + 4);
+                s += qa[0] * lo_f(kv.x) + qa[1] * hi_f(kv.x) + qa[2] * lo_f(kv.y) + qa[3] * hi_f(kv.y) +
+                     qb[0] * lo_f(kv.z) + qb[1] * hi_f(kv.z) + qb[2] * lo_f(kv.w) + qb[3] * hi_f(kv.w);
+              }
+            } else {
+              for (int i = 0; i < D; ++i) s += qg[i] * ldf(kr + i);
             }
           } else {
-            for (int i = 0; i < D; ++i) s += qg[i] * ldf(kr + i);
-          }
-        } else {
-          if ((D & 3) == 0) {
-            for (int i = 0; i < D; i += 4) {
-              const f32x4 kv = *reinterpret_cast<const f32x4*>(kr + i);
-              const f32x4 qa = *reinterpret_cast<const f32x4*>(qg + i);
-              s += qa[0] * kv[0] + qa[1] * kv[1] + qa[2] * kv[2] + qa[3] * kv[3];
+            if ((D & 3) == 0) {
+              for (int i = 0; i < D; i += 4) {
+                const f32x4 kv = *reinterpret_cast<const f32x4*>(kr + i);
+                const f32x4 qa = *reinterpret_cast<const f32x4*>(qg + i);
+                s += qa[0] * kv[0] + qa[1] * kv[1] + qa[2] * kv[2] + qa[3] * kv[3];
+              }
+            } else {
+              for (int i = 0; i < D; ++i) s += qg[i] * ldf(kr + i);
             }
-          } else {
-            for (int i = 0; i < D; ++i) s += qg[i] * ldf(kr + i);
           }
+          s *= a.scale;
         }
-        s *= a.scale;
+        sc[it] = s;
       }
-      sc[it] = s;
-    }
-    __syncthreads();
-    for (int r = wave; r < rep; r += NW) {      // the tile's place in head r's running softmax
-      const float s = sc[r * KT + lane];
-      const float mo = s_m[r];
-      const float m = fmaxf(mo, wave_max(s));   // finite: a tile holds at least one key
-      const float e = s == -INFINITY ? 0.f : expf(s - m);
-      const float sum = wave_sum(e);
-      sc[r * KT + lane] = e;
-      if (lane == 0) {
-        const float corr = mo == -INFINITY ? 0.f : expf(mo - m);
-        s_c[r] = corr;
-        s_l[r] = s_l[r] * corr + sum;
-        s_m[r] = m;
+      __syncthreads();
+      for (int r = wave; r < rep; r += NW) {      // the tile's place in head r's running softmax
+        const float s = sc[r * KT + lane];
+        const float mo = s_m[r];
+        const float m = fmaxf(mo, wave_max(s));   // finite: a tile holds at least one position of its span
+        const float e = s == -INFINITY ? 0.f : expf(s - m);
+        const float sum = wave_sum(e);
+        sc[r * KT + lane] = e;
+        if (lane == 0) {
+          const float corr = mo == -INFINITY ? 0.f : expf(mo - m);
+          s_c[r] = corr;
+          s_l[r] = s_l[r] * corr + sum;
+          s_m[r] = m;
+        }
       }
-    }
-    __syncthreads();
+      __syncthreads();
+      const int j0 = max(sa - pos0, 0), j1 = min(sb - pos0, KT);   // the tile's positions inside the span
 #pragma unroll
-    for (int u = 0; u < MAX_ACC; ++u) {
-      const int i = threadIdx.x + u * NT;
-      if (i < RV) {
-        const int r = i / Dv, d = i % Dv;
-        const float* wr = sc + r * KT;
-        float s = acc[u] * s_c[r];
-        for (int j = 0; j < nk; ++j) s += wr[j] * ldf(v_cache + (size_t)s_row[j] * Dv + d);
-        acc[u] = s;
+      for (int u = 0; u < MAX_ACC; ++u) {
+        const int i = threadIdx.x + u * NT;
+        if (i < RV) {
+          const int r = i / Dv, d = i % Dv;
+          const float* wr = sc + r * KT;
+          float s = acc[u] * s_c[r];
+          if (sizeof(AT) == 2 && BS == 16) {     // a page's 16 values of entry d: two 16-byte loads
+            for (int pg = j0 / 16; pg * 16 < j1; ++pg) {
+              const uint4* vp = reinterpret_cast<const uint4*>(v_cache + ((size_t)s_page[pg] * Dv + d) * 16);
+              const uint4 va = vp[0], vb = vp[1];
+              const uint32_t w8[8] = {va.x, va.y, va.z, va.w, vb.x, vb.y, vb.z, vb.w};
+              const float* wp = wr + pg * 16;
+#pragma unroll
+              for (int k = 0; k < 8; ++k) {      // a weight of 0 (outside the span) takes nothing from its slot
+                const float w0 = wp[2 * k], w1 = wp[2 * k + 1];
+                s += w0 != 0.f ? w0 * lo_f(w8[k]) : 0.f;
+                s += w1 != 0.f ? w1 * hi_f(w8[k]) : 0.f;
+              }
+            }
+          } else {
+            for (int j = j0; j < j1; ++j) s += wr[j] * ldf(v_cache + ((size_t)s_page[j / BS] * Dv + d) * BS + j % BS);
+          }
+          acc[u] = s;
+        }
       }
     }
   }
@@ -206,7 +214,7 @@ extern "C" int ka_rope_append(void* q_out, const void* qkv, const float* inv_fre
   KA_CHECK_LAUNCH();
 }
 
-// mode 0: the fastest kernel the shape allows; 1: the vector kernel
+// mode: the longest run of rows that one sequence brings to the step, or 0 to ask for the vector kernel
 extern "C" int ka_sliding_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
                                     const int* block_tables, const int* q_starts, int num_seqs, const int* positions,
                                     const int* slots, const void* gate, int gs, int g_off, int T, int H, int G, int D,
@@ -216,11 +224,17 @@ extern "C" int ka_sliding_attention(void* out, const void* q, const void* k_cach
   if (H <= 0 || G <= 0 || H % G || H / G > MAX_REP || (H / G) * Dv > NT * MAX_ACC || D <= 0 || Dv <= 0 || BS <= 0 ||
       window < 0 || keep_first < 0 || num_seqs <= 0)
     return (int)hipErrorInvalidValue;
-  (void)mode;
+  if (KT % BS) return (int)hipErrorInvalidValue;   // tiles are whole pages
+  if (q_starts == nullptr && T > num_seqs) return (int)hipErrorInvalidValue;   // row t reads block-table row t
+  SlideArgs a{block_tables, q_starts, positions, slots, num_seqs, H, G, D, Dv, window, keep_first, BS, max_blocks, gs, g_off, scale};
+  // prompt portions in bf16 go to the matrix cores; mode = the longest run of rows of one sequence in the step
+  // (0: decode rows only, or the vector kernel is asked for)
+  if (!f32 && mode >= TILE_MIN_ROWS && q_starts != nullptr && ka_sliding_attention_tile_ok(H, G, D, Dv, BS))
+    return sliding_attention_tile((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
+                                  (const bf16_t*)gate, a, mode, st);
   const int rep = H / G;
   const size_t lds = (size_t)(rep * D + rep * KT) * sizeof(float);
   if (lds > 60 * 1024) return (int)hipErrorInvalidValue;
-  SlideArgs a{block_tables, q_starts, positions, slots, num_seqs, H, G, D, Dv, window, keep_first, BS, max_blocks, gs, g_off, scale};
   if (lds > 48 * 1024) {
     const void* fn = f32 ? reinterpret_cast<const void*>(sliding_attention_kernel<float>)
                          : reinterpret_cast<const void*>(sliding_attention_kernel<bf16_t>);

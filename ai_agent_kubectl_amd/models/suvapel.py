@@ -20,7 +20,7 @@ Mixers (activations in the engine dtype, bf16 or fp32; what is marked fp32 is fp
   parallel          left_scale * attention + right_scale * delta rule, both on h.
 Feed-forward: down(silu(gate h + b) * (up h + b)) + b.
 
-Cache: per attention layer K [NB, G, BS, D] and V [NB, G, BS, Dv] under the engine's single block table.  State:
+Cache: per attention layer K [NB, G, BS, D] and V [NB, G, Dv, BS] (a page's values of one entry contiguous) under the engine's single block table.  State:
 per layer and state slot the delta-rule memory [H, Dv, D] fp32 and the convolutions' last taps - 1 inputs (engine
 dtype), indexed by the sequence's state slot (`AttnMeta.state_slots`); a row at position 0 starts from zeros, so
 slots are reused without clearing.  Prefill, chunked prefill, mixed and decode steps all run this forward; the
@@ -81,7 +81,7 @@ class SuvapelModel:
 
     # ---- the runner's model interface ----------------------------------------------------------
     def alloc_cache(self, num_blocks: int, block_size: int):
-        """(k_cache, v_cache): per layer [NB, G, BS, D] / [NB, G, BS, Dv] for its attention half (None without one)."""
+        """(k_cache, v_cache): per layer [NB, G, BS, D] / [NB, G, Dv, BS] for its attention half (None without one)."""
         ks: List[Optional[torch.Tensor]] = []
         vs: List[Optional[torch.Tensor]] = []
         for L in self.cfg.layers:
@@ -92,7 +92,7 @@ class SuvapelModel:
             else:
                 z = dict(dtype=self.dtype, device=self.device)
                 ks.append(torch.zeros((num_blocks, a.kv_heads, block_size, a.dim), **z))
-                vs.append(torch.zeros((num_blocks, a.kv_heads, block_size, a.vdim), **z))
+                vs.append(torch.zeros((num_blocks, a.kv_heads, a.vdim, block_size), **z))
         return ks, vs
 
     def alloc_state(self, num_slots: int) -> None:
@@ -144,7 +144,7 @@ class SuvapelModel:
         q = mixers.rope_append(cv, L.get("inv_freq"), L["rot_mag"], meta.positions, meta.slot_mapping, k_cache, v_cache,
                                a.heads, a.kv_heads, a.dim, a.vdim, a.rot.dims)
         o = mixers.sliding_attention(q, k_cache, v_cache, meta.block_tables, qs, meta.positions, meta.slot_mapping, proj,
-                                     col["att_g"], a.window, a.keep_first, a.scale)
+                                     col["att_g"], a.window, a.keep_first, a.scale, meta.max_q_len, meta.num_decode)
         return F.linear(o, L["att_wo"])
 
     # ---- forward -------------------------------------------------------------------------------

@@ -138,6 +138,7 @@ _MIX_SIGS = {
     "ka_short_conv": [P, P, I, I, I, P, I, P, P, P, I, P, I, I, I, P],
     "ka_rope_append": [P, P, P, F, P, P, P, P, I, I, I, I, I, I, I, I, P],
     "ka_sliding_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, I, I, F, I, I, P],
+    "ka_sliding_attention_tile_ok": [I, I, I, I, I],
     "ka_delta_prep": [P, P, P, P, I, P, I, I, P, I, I, P, P, I, I, I, I, I, I, P],
     "ka_delta_scan": [P, P, P, I, I, P, P, P, P, P, I, P, I, I, I, I, I, I, P],
 }

@@ -559,13 +559,14 @@ def rope_append(qkv: torch.Tensor, inv_freq: Optional[torch.Tensor], mag: float,
                 rot: int) -> torch.Tensor:
     """Rows [q (H x D) | k (G x D) | v (G x Dv)] -> q [T, H, D] with rotary positions on the first `rot` entries of
     each head (pairs (i, i + rot/2), angle = position * inv_freq[i] in fp32, cos and sin times `mag`); the rotated
-    keys and the values are appended to the paged cache [NB, G, BS, D] / [NB, G, BS, Dv] at `slots` (-1: skipped)."""
+    keys and the values are appended to the paged cache [NB, G, BS, D] / [NB, G, Dv, BS] at `slots` (-1: skipped)."""
     if _ref(qkv):
         return ref.rope_append(qkv, inv_freq, mag, positions, slots, k_cache, v_cache, H, G, D, Dv, rot)
     lib = require_mixers()
     T = qkv.shape[0]
     assert qkv.is_contiguous() and qkv.shape[1] == (H + G) * D + G * Dv and k_cache.dtype == qkv.dtype == v_cache.dtype
-    assert k_cache.shape[1:] == (G, k_cache.shape[2], D) and v_cache.shape == (k_cache.shape[0], G, k_cache.shape[2], Dv)
+    assert k_cache.shape[1:] == (G, k_cache.shape[2], D) and v_cache.shape == (k_cache.shape[0], G, Dv, k_cache.shape[2])
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
     assert positions.dtype == torch.int32 and slots.dtype == torch.int32 and positions.shape[0] >= T and slots.shape[0] >= T
     assert rot == 0 or (inv_freq.dtype == torch.float32 and inv_freq.numel() * 2 == rot and rot <= D)
     q = torch.empty((T, H, D), dtype=qkv.dtype, device=qkv.device)
@@ -574,23 +575,27 @@ def rope_append(qkv: torch.Tensor, inv_freq: Optional[torch.Tensor], mag: float,
     return q
 
 
-SLIDING_TILE = True   # bf16 sliding attention on the matrix cores where the shape allows (False: the vector kernel)
+SLIDING_TILE = True   # bf16 prompt portions of sliding attention on the matrix cores where the shape allows
 
 
 def sliding_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                       q_starts: Optional[torch.Tensor], positions: torch.Tensor, slots: torch.Tensor,
-                      gate_src: Optional[torch.Tensor], g_off: int, window: int, keep_first: int, scale: float) -> torch.Tensor:
-    """Softmax attention with grouped keys / values over a paged cache: the query at position p sees the keys
-    j <= p with p - j < window or j < keep_first (window 0: all of 0 .. p; kept keys stay at their own positions).
-    Head h's result is multiplied by sigmoid(gate_src[t, g_off + h]) (gate_src None: no gate).
-    q [T, H, D] -> [T, H * Dv].  q_starts None: row t is block-table row t (a decode step)."""
+                      gate_src: Optional[torch.Tensor], g_off: int, window: int, keep_first: int, scale: float,
+                      max_q: int = 0, num_decode: int = 0) -> torch.Tensor:
+    """Softmax attention with grouped keys / values over a paged cache (k_cache [NB, G, BS, D], v_cache
+    [NB, G, Dv, BS]): the query at position p sees the keys j <= p with p - j < window or j < keep_first (window 0:
+    all of 0 .. p; kept keys stay at their own positions).  Head h's result is multiplied by
+    sigmoid(gate_src[t, g_off + h]) (gate_src None: no gate).  q [T, H, D] -> [T, H * Dv].
+    q_starts None: row t is block-table row t (a decode step).  max_q: the longest run of rows of one sequence in a
+    varlen step (0: unknown), num_decode: its leading one-row sequences; they choose the kernel, not the result."""
     if _ref(q):
         return ref.sliding_attention(q, k_cache, v_cache, block_tables, q_starts, positions, slots, gate_src, g_off,
                                      window, keep_first, scale)
     lib = require_mixers()
     T, H, D = q.shape
-    G, BS, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    G, BS, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
     assert q.is_contiguous() and k_cache.dtype == q.dtype == v_cache.dtype and k_cache.shape[3] == D and H % G == 0
+    assert v_cache.shape == (k_cache.shape[0], G, Dv, BS) and k_cache.is_contiguous() and v_cache.is_contiguous()
     assert block_tables.dtype == torch.int32 and block_tables.is_contiguous() and block_tables.dim() == 2
     assert positions.dtype == torch.int32 and slots.dtype == torch.int32 and positions.shape[0] >= T and slots.shape[0] >= T
     assert q_starts is None or (q_starts.dtype == torch.int32 and q_starts.shape[0] == block_tables.shape[0] + 1)
@@ -600,11 +605,25 @@ def sliding_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         assert gate_src.dtype == q.dtype and gate_src.is_contiguous() and gate_src.shape[0] >= T
         gs = gate_src.shape[1]
         assert 0 <= g_off and g_off + H <= gs
+    def tail(rows):
+        return (_p(positions), _p(slots), _p(gate_src), gs, g_off, rows, H, G, D, Dv, int(window), int(keep_first), BS,
+                block_tables.shape[1], float(scale), _f32(q))
+
+    if (SLIDING_TILE and q_starts is not None and max_q >= 8 and q.dtype == torch.bfloat16
+            and lib.ka_sliding_attention_tile_ok(H, G, D, Dv, BS)):
+        # rows past the last sequence (a padded step) belong to no tile and stay zero
+        out = torch.zeros((T, H * Dv), dtype=q.dtype, device=q.device)
+        nd = min(int(num_decode), block_tables.shape[0])
+        if nd > 0:   # the leading one-row sequences: rows 0 .. nd - 1 only, row t is block-table row t, through the vector kernel
+            check(lib.ka_sliding_attention(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), None, nd, *tail(nd), 0,
+                                           _stream()), "sliding_attention")
+        if block_tables.shape[0] > nd:   # (q_starts holds absolute rows, so the remaining sequences index q and out as they are)
+            check(lib.ka_sliding_attention(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables[nd:]), _p(q_starts[nd:]),
+                                           block_tables.shape[0] - nd, *tail(T), int(max_q), _stream()), "sliding_attention_tile")
+        return out
     out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
     check(lib.ka_sliding_attention(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(q_starts),
-                                   block_tables.shape[0], _p(positions), _p(slots), _p(gate_src), gs, g_off, T, H, G, D, Dv,
-                                   int(window), int(keep_first), BS, block_tables.shape[1], float(scale), _f32(q),
-                                   0 if SLIDING_TILE else 1, _stream()), "sliding_attention")
+                                   block_tables.shape[0], *tail(T), 0, _stream()), "sliding_attention")
     return out
 
 

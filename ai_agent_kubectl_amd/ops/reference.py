@@ -490,7 +490,7 @@ def short_conv(proj, off: int, C: int, w, state, seq_slots, q_starts, positions,
 def rope_append(qkv, inv_freq, mag: float, positions, slots, k_cache, v_cache, H: int, G: int, D: int, Dv: int, rot: int):
     """Rows [q (H x D) | k (G x D) | v (G x Dv)]: rotary positions (angle = position * inv_freq, cos and sin times
     mag) on the first `rot` entries of every q and k head; -> q [T, H, D]; k and v go to the paged cache
-    [NB, G, BS, D] / [NB, G, BS, Dv] at `slots`."""
+    [NB, G, BS, D] / [NB, G, Dv, BS] at `slots`."""
     T = qkv.shape[0]
     q = qkv[:, :H * D].float().view(T, H, D)
     k = qkv[:, H * D:(H + G) * D].float().view(T, G, D)
@@ -510,7 +510,7 @@ def rope_append(qkv, inv_freq, mag: float, positions, slots, k_cache, v_cache, H
     if ok.any():
         bs = k_cache.shape[2]
         k_cache[sl[ok] // bs, :, sl[ok] % bs] = k[ok].to(k_cache.dtype)
-        v_cache[sl[ok] // bs, :, sl[ok] % bs] = v[ok].to(v_cache.dtype)
+        v_cache[sl[ok] // bs, :, :, sl[ok] % bs] = v[ok].to(v_cache.dtype)
     return q.to(qkv.dtype).contiguous()
 
 
@@ -519,7 +519,7 @@ def sliding_attention(q, k_cache, v_cache, block_tables, q_starts, positions, sl
     """q [T, H, D] -> [T, H * Dv]: softmax attention over the keys j <= p with p - j < window or j < keep_first
     (window 0: all); head h's result times sigmoid(gate_src[t, g_off + h]) (gate_src None: no gate)."""
     T, H, D = q.shape
-    G, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    G, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
     rep = H // G
     out = torch.zeros(T, H * Dv, dtype=q.dtype, device=q.device)
     pos_l, slot_l = positions.tolist(), slots.tolist()
@@ -532,7 +532,7 @@ def sliding_attention(q, k_cache, v_cache, block_tables, q_starts, positions, sl
             js = torch.cat([torch.arange(0, min(keep_first, lo)), torch.arange(lo, p + 1)])
             pages = block_tables[i].long()[js // bs]
             k = k_cache[pages, :, js % bs, :].float().repeat_interleave(rep, dim=1)   # [n, H, D]
-            v = v_cache[pages, :, js % bs, :].float().repeat_interleave(rep, dim=1)
+            v = v_cache[pages, :, :, js % bs].float().repeat_interleave(rep, dim=1)   # [n, H, Dv]
             w = torch.softmax(torch.einsum("hd,nhd->hn", q[t].float(), k) * scale, dim=1)
             o = torch.einsum("hn,nhd->hd", w, v)
             if gate_src is not None:

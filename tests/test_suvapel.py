@@ -250,7 +250,7 @@ class Paged:
         nb = sum(need) + 3
         perm = torch.randperm(nb, generator=torch.Generator().manual_seed(seed)).tolist()
         self.k = torch.full((nb, G, BS, D), 7.0, dtype=dtype, device=device)       # whatever a page held before
-        self.v = torch.full((nb, G, BS, Dv), -7.0, dtype=dtype, device=device)
+        self.v = torch.full((nb, G, Dv, BS), -7.0, dtype=dtype, device=device)
         self.tables = torch.zeros((len(lens), max(need)), dtype=torch.int32)
         for i, n in enumerate(need):
             self.tables[i, :n] = torch.tensor([perm.pop() for _ in range(n)], dtype=torch.int32)
@@ -278,7 +278,7 @@ def _attend(device, q, k, v, m, cuts, gate=None, dtype=torch.float32):
         decode = c == 1 and at > 0
         gs = gate[at:at + c].contiguous().to(dtype).to(device) if gate is not None else None
         out.append(mixers.sliding_attention(qq, pg.k, pg.v, pg.tables.to(device), None if decode else _seq_meta([c], device), p, sl,
-                                            gs, 2 if gate is not None else 0, m["window"], m["keep_first"], m["scale"]))
+                                            gs, 2 if gate is not None else 0, m["window"], m["keep_first"], m["scale"], max_q=c))
         at += c
     return torch.cat(out)
 
@@ -653,3 +653,79 @@ def test_graph_decode_matches_eager(tmp_path, dtype):
         if graphs:
             assert eng.runner.stats["graph_replays"] > 0
     assert got[0] == got[1]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,Dv,window,keep", [(4, 1, 64, 64, 44, 7), (6, 2, 64, 128, 36, 5), (8, 2, 128, 128, 100, 20), (2, 2, 128, 64, 0, 0),
+                                                  (8, 1, 256, 256, 17, 33), (4, 4, 64, 256, 1, 0), (3, 1, 128, 128, 16, 16)])
+def test_sliding_attention_matrix_core_kernel(H, G, D, Dv, window, keep):
+    """bf16 prompt portions run on the matrix cores: against the oracle on the bf16-rounded inputs, whole and in
+    portions whose rows start anywhere in a page; the vector kernel agrees."""
+    from ai_agent_kubectl_amd.ops import mixers
+
+    g = torch.Generator().manual_seed(H + D + window)
+    T = 150
+    bf = lambda t: t.to(torch.bfloat16).float()
+    q, k, v = bf(torch.randn(T, H, D, generator=g)), bf(torch.randn(T, G, D, generator=g)), bf(torch.randn(T, G, Dv, generator=g))
+    gate = bf(torch.randn(T, H + 5, generator=g) * 2)
+    m = dict(window=window, keep_first=keep, scale=D ** -0.5 * 2)
+    want = oracle.window_attention(q.double().numpy(), k.double().numpy(), v.double().numpy(), m["scale"], window or T + 1, keep)
+    want = (want * oracle.sigmoid(gate.double().numpy()[:, 2:2 + H])[:, :, None]).reshape(T, H * Dv)
+    assert mixers.require_mixers().ka_sliding_attention_tile_ok(H, G, D, Dv, BS)
+    outs = []
+    for tile in (True, False):
+        mixers.SLIDING_TILE = tile
+        try:
+            for cuts in ([T], [37, 9, 70, 1, 33], [16, 16, 8, 110]):
+                got = _attend("cuda", q, k, v, m, cuts, gate, dtype=torch.bfloat16)
+                assert close(got, want, 2e-2, 2e-2), (tile, cuts)
+                outs.append(got.float().cpu())
+        finally:
+            mixers.SLIDING_TILE = True
+    assert (outs[0] - outs[3]).abs().max() < 2e-2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("key,seen", [(140 - 43, True), (140 - 44, False), (6, True), (7, False), (0, True)])
+def test_window_edges_on_the_matrix_cores(key, seen):
+    """Window 44, first 7 tokens kept, the query at position 140 inside a 150-row prompt portion (bf16, head size 64):
+    the key whose score stands out carries the result exactly when the mask lets it."""
+    g = torch.Generator().manual_seed(key)
+    T, D, Dv, qpos = 150, 64, 64, 140
+    q, k, v = torch.randn(T, 2, D, generator=g) * 0.05, torch.randn(T, 1, D, generator=g) * 0.05, torch.randn(T, 1, Dv, generator=g)
+    q[qpos], k[key] = 0.0, 0.0
+    q[qpos, :, 0], k[key, 0, 0] = 8.0, 8.0
+    v[key, 0] = 100.0
+    m = dict(window=44, keep_first=7, scale=1.0)
+    out = _attend("cuda", q, k, v, m, [T], dtype=torch.bfloat16)[qpos].float().cpu()
+    assert (abs(float(out[0]) - 100.0) < 2.0) == seen and (abs(float(out[Dv]) - 100.0) < 2.0) == seen
+
+
+@pytest.mark.gpu
+def test_mixed_steps_on_the_matrix_cores(tmp_path):
+    """bf16 engine with head sizes the matrix-core attention takes: single decoded rows of two requests ahead of a
+    prompt portion of a third in one step (the decoded rows go through the vector kernel, the portion through the
+    tile kernel), then the roles change."""
+    c = make_config([parallel_layer(left=attention_cfg(heads=4, kv_heads=2, dim=64, vdim=64, window=24, keep_first=3, rot_dims=32),
+                                    right=delta_mixer_cfg(heads=2, kv_heads=1, dim=32, vdim=32, conv=4), ff=64), delta_layer(ff=32)],
+                    width=64, vocab=128, side=8)
+    W = oracle.random_tensors(c, 21)
+    path = write_checkpoint(tmp_path / "mixed", c, W)
+    toks = {k: tokens_for(c, n, seed=50 + n) for k, n in (("a", 44), ("b", 37), ("c", 90))}
+    want = {k: want_logits(c, W, v) for k, v in toks.items()}
+    sess = session(path, "cuda", dtype="bfloat16", max_tokens=256)
+    plan = [[("a", 40), ("b", 35)], [("a", 1), ("b", 1), ("c", 50)], [("a", 1), ("c", 1), ("b", 1)], [("c", 37), ("a", 1)],
+            [("c", 1), ("a", 1)], [("c", 1)]]
+    at, got = {k: 0 for k in toks}, {k: [] for k in toks}
+    for step in plan:
+        entries = []
+        for rid, n in step:
+            entries.append({"id": rid, "tokens": toks[rid][at[rid]:at[rid] + n], "want": list(range(n))})
+            at[rid] += n
+        out = sess.step(entries, [rid for rid, _ in step if at[rid] == len(toks[rid])])
+        o = 0
+        for e in entries:
+            got[e["id"]].append(out[o:o + len(e["tokens"])])
+            o += len(e["tokens"])
+    for k in toks:
+        assert at[k] == len(toks[k]) and rel_err(np.concatenate(got[k]), want[k]) < tol("bfloat16"), k
