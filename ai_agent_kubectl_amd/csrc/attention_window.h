@@ -19,4 +19,4 @@ struct SlideArgs {
 // the matrix-core kernel (bf16): 1 if it takes the shape
 extern "C" int ka_sliding_attention_tile_ok(int H, int G, int D, int Dv, int BS);
 int sliding_attention_tile(bf16_t* out, const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const bf16_t* gate,
-                           const SlideArgs& a, int max_q, hipStream_t st);
+                           const SlideArgs& a, int max_q, int rows_, hipStream_t st);

@@ -214,7 +214,7 @@ extern "C" int ka_rope_append(void* q_out, const void* qkv, const float* inv_fre
   KA_CHECK_LAUNCH();
 }
 
-// mode: the longest run of rows that one sequence brings to the step, or 0 to ask for the vector kernel
+// mode: the longest run of rows that one sequence brings to the step (1 for single rows), or 0 to ask for the vector kernel
 extern "C" int ka_sliding_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
                                     const int* block_tables, const int* q_starts, int num_seqs, const int* positions,
                                     const int* slots, const void* gate, int gs, int g_off, int T, int H, int G, int D,
@@ -227,11 +227,11 @@ extern "C" int ka_sliding_attention(void* out, const void* q, const void* k_cach
   if (KT % BS) return (int)hipErrorInvalidValue;   // tiles are whole pages
   if (q_starts == nullptr && T > num_seqs) return (int)hipErrorInvalidValue;   // row t reads block-table row t
   SlideArgs a{block_tables, q_starts, positions, slots, num_seqs, H, G, D, Dv, window, keep_first, BS, max_blocks, gs, g_off, scale};
-  // prompt portions in bf16 go to the matrix cores; mode = the longest run of rows of one sequence in the step
-  // (0: decode rows only, or the vector kernel is asked for)
-  if (!f32 && mode >= TILE_MIN_ROWS && q_starts != nullptr && ka_sliding_attention_tile_ok(H, G, D, Dv, BS))
+  // bf16 on the matrix cores where the shape allows: prompt portions (mode = the longest run of rows of one
+  // sequence in the step) and single rows (q_starts null); mode 0 asks for the vector kernel
+  if (!f32 && mode > 0 && (q_starts == nullptr || mode >= TILE_MIN_ROWS) && ka_sliding_attention_tile_ok(H, G, D, Dv, BS))
     return sliding_attention_tile((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
-                                  (const bf16_t*)gate, a, mode, st);
+                                  (const bf16_t*)gate, a, mode, T, st);
   const int rep = H / G;
   const size_t lds = (size_t)(rep * D + rep * KT) * sizeof(float);
   if (lds > 60 * 1024) return (int)hipErrorInvalidValue;

@@ -35,29 +35,49 @@ KA_DEV void split2(const f32x4& p, s16x4& hi, s16x4& lo) {
   }
 }
 
-template <int DK, int DB>   // D = 32 DK, Dv = 16 DB
+// DEC false: a prompt portion.  The 16 query columns of a wave are 16 consecutive rows of one sequence for one query
+//   head; the workgroup's waves are the heads of the key/value group.
+// DEC true: single rows (a decode step, or the one-row sequences of a mixed step).  The query columns are the H / G
+//   heads of the key/value group for ONE row, so a page is read once for all of them; the workgroup's four waves
+//   take every fourth step of the pages with a softmax of their own and are merged through LDS at the end.
+template <int DK, int DB, bool DEC>   // D = 32 DK, Dv = 16 DB
 __global__ __launch_bounds__(512) void sliding_tile_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
-                                                            const bf16_t* __restrict__ k_cache,
-                                                            const bf16_t* __restrict__ v_cache,
-                                                            const bf16_t* __restrict__ gate, SlideArgs a, int tiles_per_seq) {
+                                                           const bf16_t* __restrict__ k_cache,
+                                                           const bf16_t* __restrict__ v_cache,
+                                                           const bf16_t* __restrict__ gate, SlideArgs a, int tiles_per_seq) {
   constexpr int D = 32 * DK, Dv = 16 * DB;
-  const int seq = blockIdx.x / tiles_per_seq, tile = blockIdx.x % tiles_per_seq;
-  const int r0 = a.q_starts[seq] + tile * 16, r1 = a.q_starts[seq + 1];
-  if (r0 >= r1) return;
-  const int nrows = min(16, r1 - r0);
-  const int g = blockIdx.y, H = a.H, G = a.G;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  extern __shared__ float lds[];   // DEC: [nw][rep] maxima, [nw][rep] sums, [nw][rep][Dv] partial results
+  const int g = blockIdx.y, H = a.H, G = a.G, rep = H / G;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
-  const int h = g * (H / G) + wave;
+  int seq, r0, nq, P0, p_last;
+  if constexpr (DEC) {
+    seq = r0 = blockIdx.x;                         // row t is block-table row t
+    nq = rep;
+    if (a.slots[r0] < 0) {                         // a padding row
+      for (int i = threadIdx.x; i < rep * Dv; i += blockDim.x) out[((size_t)r0 * H + g * rep) * Dv + i] = 0;
+      return;
+    }
+    P0 = p_last = a.positions[r0];
+  } else {
+    seq = blockIdx.x / tiles_per_seq;
+    r0 = a.q_starts[seq] + (blockIdx.x % tiles_per_seq) * 16;
+    const int r1 = a.q_starts[seq + 1];
+    if (r0 >= r1) return;
+    nq = min(16, r1 - r0);
+    P0 = a.positions[r0];                          // the rows' positions are P0, P0 + 1, ...
+    p_last = P0 + nq - 1;
+  }
   const int* bt = a.block_tables + (size_t)seq * a.max_blocks;
-  const int P0 = a.positions[r0];                 // the rows' positions are P0, P0 + 1, ...
-  const int p_last = P0 + nrows - 1;
   const int W = a.window > 0 ? a.window : 0x3fffffff;
-  const bool valid_q = col < nrows;
-  const int p_q = P0 + col;                       // this lane's query position
+  const bool valid_q = col < nq;
+  const int cq = min(col, nq - 1);
+  const int p_q = DEC ? P0 : P0 + col;             // this lane's query position
+  const int row_q = DEC ? r0 : r0 + cq;            // its row of q / gate / out
+  const int h_q = g * rep + (DEC ? cq : wave);     // its query head
   bf16x8 qf[DK];
   {
-    const bf16_t* qp = q + ((size_t)(r0 + min(col, nrows - 1)) * H + h) * D + 8 * grp;
+    const bf16_t* qp = q + ((size_t)row_q * H + h_q) * D + 8 * grp;
 #pragma unroll
     for (int kk = 0; kk < DK; ++kk) qf[kk] = as_bf16x8(*reinterpret_cast<const uint4*>(qp + 32 * kk));
   }
@@ -70,7 +90,7 @@ __global__ __launch_bounds__(512) void sliding_tile_kernel(bf16_t* __restrict__ 
   f32x4 O[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db) O[db] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int i0 = 0; i0 < total; i0 += NP) {
+  for (int i0 = DEC ? wave * NP : 0; i0 < total; i0 += DEC ? nw * NP : NP) {
     f32x4 sv[NP];
     int pbase[NP], pgs[NP];
     float mt = -INFINITY;
@@ -145,28 +165,77 @@ __global__ __launch_bounds__(512) void sliding_tile_kernel(bf16_t* __restrict__ 
   }
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
-  float fin = valid_q ? 1.0f / l_run : 0.f;
-  if (gate != nullptr && valid_q) fin *= 1.0f / (1.0f + __expf(-bf2f(gate[(size_t)(r0 + col) * a.gs + a.g_off + h])));
-  float fr[4];
+  if constexpr (DEC) {
+    // merge the waves' partial softmaxes: out = sum_w O_w e^(m_w - M) / sum_w l_w e^(m_w - M)
+    float* sm = lds;                     // [nw][rep]
+    float* sl = sm + nw * rep;           // [nw][rep]
+    float* so = sl + nw * rep;           // [nw][rep][Dv]
+    if (grp == 0 && col < rep) {
+      sm[wave * rep + col] = m_run;
+      sl[wave * rep + col] = l_run;
+    }
 #pragma unroll
-  for (int r = 0; r < 4; ++r) fr[r] = __shfl(fin, 4 * grp + r, 64);
+    for (int r = 0; r < 4; ++r) {
+      const int hq = 4 * grp + r;
+      if (hq < rep) {
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int row = 4 * grp + r;
-    if (row < nrows) {
-      bf16_t* op = out + ((size_t)(r0 + row) * H + h) * Dv + col;
+        for (int db = 0; db < DB; ++db) so[((size_t)wave * rep + hq) * Dv + 16 * db + col] = O[db][r];
+      }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < rep * Dv; i += blockDim.x) {
+      const int hq = i / Dv, d = i % Dv;
+      float M = -INFINITY;
+      for (int w = 0; w < nw; ++w) M = fmaxf(M, sm[w * rep + hq]);
+      float num = 0.f, den = 0.f;
+      for (int w = 0; w < nw; ++w) {
+        const float mw = sm[w * rep + hq];
+        const float f = mw == -INFINITY ? 0.f : __expf(mw - M);
+        num += so[((size_t)w * rep + hq) * Dv + d] * f;
+        den += sl[w * rep + hq] * f;
+      }
+      float o = num / den;
+      if (gate != nullptr) o *= 1.0f / (1.0f + __expf(-bf2f(gate[(size_t)r0 * a.gs + a.g_off + g * rep + hq])));
+      out[((size_t)r0 * H + g * rep + hq) * Dv + d] = f2bf(o);
+    }
+  } else {
+    float fin = valid_q ? 1.0f / l_run : 0.f;
+    if (gate != nullptr && valid_q) fin *= 1.0f / (1.0f + __expf(-bf2f(gate[(size_t)row_q * a.gs + a.g_off + h_q])));
+    float fr[4];
 #pragma unroll
-      for (int db = 0; db < DB; ++db) op[16 * db] = f2bf(O[db][r] * fr[r]);
+    for (int r = 0; r < 4; ++r) fr[r] = __shfl(fin, 4 * grp + r, 64);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = 4 * grp + r;
+      if (row < nq) {
+        bf16_t* op = out + ((size_t)(r0 + row) * H + h_q) * Dv + col;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) op[16 * db] = f2bf(O[db][r] * fr[r]);
+      }
     }
   }
 }
 
+constexpr int DEC_WAVES = 4;
+
 template <int DK, int DB>
 int launch_tile(bf16_t* out, const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const bf16_t* gate,
-                const SlideArgs& a, int max_q, hipStream_t st) {
-  const int tiles = (max_q + 15) / 16;
-  sliding_tile_kernel<DK, DB><<<dim3(a.num_seqs * tiles, a.G), 64 * (a.H / a.G), 0, st>>>(out, q, k_cache, v_cache, gate, a,
-                                                                                        tiles);
+                const SlideArgs& a, int max_q, int rows_, hipStream_t st) {
+  if (a.q_starts == nullptr) {   // single rows
+    const int rep = a.H / a.G;
+    const size_t lds = (size_t)(DEC_WAVES * rep * (2 + 16 * DB)) * sizeof(float);
+    if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
+    if (lds > 48 * 1024) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(sliding_tile_kernel<DK, DB, true>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return (int)e;
+    }
+    sliding_tile_kernel<DK, DB, true><<<dim3(rows_, a.G), 64 * DEC_WAVES, lds, st>>>(out, q, k_cache, v_cache, gate, a, 1);
+  } else {
+    const int tiles = (max_q + 15) / 16;
+    sliding_tile_kernel<DK, DB, false><<<dim3(a.num_seqs * tiles, a.G), 64 * (a.H / a.G), 0, st>>>(out, q, k_cache, v_cache,
+                                                                                                 gate, a, tiles);
+  }
   KA_CHECK_LAUNCH();
 }
 
@@ -177,12 +246,13 @@ extern "C" int ka_sliding_attention_tile_ok(int H, int G, int D, int Dv, int BS)
          (Dv == 64 || Dv == 128 || Dv == 256);
 }
 
-// rows of no sequence (padding after the last one) are not written: the caller clears `out`
+// q_starts set: a varlen step, `max_q` its longest run of rows; rows of no sequence (padding after the last one) are
+// not written: the caller clears `out`.  q_starts null: `rows_` single rows, row t is block-table row t.
 int sliding_attention_tile(bf16_t* out, const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const bf16_t* gate,
-                           const SlideArgs& a, int max_q, hipStream_t st) {
-  if (!ka_sliding_attention_tile_ok(a.H, a.G, a.D, a.Dv, a.BS) || max_q <= 0 || a.q_starts == nullptr)
+                           const SlideArgs& a, int max_q, int rows_, hipStream_t st) {
+  if (!ka_sliding_attention_tile_ok(a.H, a.G, a.D, a.Dv, a.BS) || (a.q_starts != nullptr ? max_q <= 0 : rows_ <= 0))
     return (int)hipErrorInvalidValue;
-#define KA_T(DK, DB) return launch_tile<DK, DB>(out, q, k_cache, v_cache, gate, a, max_q, st)
+#define KA_T(DK, DB) return launch_tile<DK, DB>(out, q, k_cache, v_cache, gate, a, max_q, rows_, st)
   if (a.D == 64) {
     if (a.Dv == 64) KA_T(2, 4);
     if (a.Dv == 128) KA_T(2, 8);

@@ -15,6 +15,10 @@
 namespace {
 using namespace rows;
 
+// elementwise row kernels: one workgroup per row when there are many rows, one entry per thread when there are few
+// (a decode step), where a thread's chain of dependent loads is the kernel's length
+inline dim3 row_grid(int rows_, int width) { return dim3(rows_, rows_ >= 1024 ? 1 : (width + NT - 1) / NT); }
+
 KA_DEV float dyt(float x, float alpha, float w, float b) { return tanhf(alpha * x) * w + b; }
 
 template <typename OT>
@@ -23,7 +27,7 @@ __global__ __launch_bounds__(NT) void dyt_norm_kernel(OT* __restrict__ out, cons
                                                       const float* __restrict__ b, int width) {
   const size_t base = (size_t)blockIdx.x * width;
   const float al = alpha[0];
-  for (int i = threadIdx.x; i < width; i += NT) stf(out + base + i, dyt(x[base + i], al, w[i], b[i]));
+  for (int i = blockIdx.y * NT + threadIdx.x; i < width; i += gridDim.y * NT) stf(out + base + i, dyt(x[base + i], al, w[i], b[i]));
 }
 
 template <typename YT, typename OT>
@@ -34,7 +38,7 @@ __global__ __launch_bounds__(NT) void residual_mix_kernel(float* __restrict__ x,
                                                           const float* __restrict__ b, int width) {
   const size_t base = (size_t)blockIdx.x * width;
   const float al = h != nullptr ? alpha[0] : 0.f;
-  for (int i = threadIdx.x; i < width; i += NT) {
+  for (int i = blockIdx.y * NT + threadIdx.x; i < width; i += gridDim.y * NT) {
     float s = c0 * ldf(y0 + base + i);
     if (y1 != nullptr) s += c1 * ldf(y1 + base + i);
     if (y2 != nullptr) s += c2 * ldf(y2 + base + i);
@@ -87,7 +91,7 @@ __global__ __launch_bounds__(NT) void silu_mul_bias_kernel(AT* __restrict__ out,
                                                            int off, int ff, const float* __restrict__ bias) {
   const AT* g = proj + (size_t)blockIdx.x * ps + off;
   AT* o = out + (size_t)blockIdx.x * ff;
-  for (int i = threadIdx.x; i < ff; i += NT) {
+  for (int i = blockIdx.y * NT + threadIdx.x; i < ff; i += gridDim.y * NT) {
     const float a = ldf(g + i) + bias[i];
     stf(o + i, a / (1.f + expf(-a)) * (ldf(g + ff + i) + bias[ff + i]));
   }
@@ -99,8 +103,8 @@ extern "C" int ka_dyt_norm(void* out, const float* x, const float* alpha, const 
                            int width, int out_f32, hipStream_t st) {
   if (rows_ <= 0) return 0;
   if (width <= 0) return (int)hipErrorInvalidValue;
-  if (out_f32) dyt_norm_kernel<float><<<rows_, NT, 0, st>>>((float*)out, x, alpha, w, b, width);
-  else dyt_norm_kernel<bf16_t><<<rows_, NT, 0, st>>>((bf16_t*)out, x, alpha, w, b, width);
+  if (out_f32) dyt_norm_kernel<float><<<row_grid(rows_, width), NT, 0, st>>>((float*)out, x, alpha, w, b, width);
+  else dyt_norm_kernel<bf16_t><<<row_grid(rows_, width), NT, 0, st>>>((bf16_t*)out, x, alpha, w, b, width);
   KA_CHECK_LAUNCH();
 }
 
@@ -110,7 +114,7 @@ extern "C" int ka_residual_mix(float* x, const void* y0, const void* y1, const v
   if (rows_ <= 0) return 0;
   if (width <= 0 || y0 == nullptr) return (int)hipErrorInvalidValue;
 #define KA_RM(YT, OT)                                                                                                  \
-  residual_mix_kernel<YT, OT><<<rows_, NT, 0, st>>>(x, (const YT*)y0, (const YT*)y1, (const YT*)y2, c0, c1, c2, (OT*)copy, \
+  residual_mix_kernel<YT, OT><<<row_grid(rows_, width), NT, 0, st>>>(x, (const YT*)y0, (const YT*)y1, (const YT*)y2, c0, c1, c2, (OT*)copy, \
                                                     (OT*)h, alpha, w, b, width)
   if (y_f32 && out_f32) KA_RM(float, float);
   else if (y_f32) KA_RM(float, bf16_t);
@@ -152,7 +156,7 @@ extern "C" int ka_silu_mul_bias(void* out, const void* proj, int ps, int off, in
                                 int f32, hipStream_t st) {
   if (rows_ <= 0) return 0;
   if (ff <= 0 || off < 0 || off + 2 * ff > ps) return (int)hipErrorInvalidValue;
-  if (f32) silu_mul_bias_kernel<float><<<rows_, NT, 0, st>>>((float*)out, (const float*)proj, ps, off, ff, bias);
-  else silu_mul_bias_kernel<bf16_t><<<rows_, NT, 0, st>>>((bf16_t*)out, (const bf16_t*)proj, ps, off, ff, bias);
+  if (f32) silu_mul_bias_kernel<float><<<row_grid(rows_, ff), NT, 0, st>>>((float*)out, (const float*)proj, ps, off, ff, bias);
+  else silu_mul_bias_kernel<bf16_t><<<row_grid(rows_, ff), NT, 0, st>>>((bf16_t*)out, (const bf16_t*)proj, ps, off, ff, bias);
   KA_CHECK_LAUNCH();
 }

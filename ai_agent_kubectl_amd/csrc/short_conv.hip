@@ -41,7 +41,7 @@ __global__ __launch_bounds__(NT) void short_conv_kernel(AT* __restrict__ out, co
   const int p = a.positions[t];
   const int taps = a.taps, C = a.C;
   const AT* st = state != nullptr ? state + (size_t)slot * (taps - 1) * C : nullptr;
-  for (int c = threadIdx.x; c < C; c += NT) {
+  for (int c = blockIdx.y * NT + threadIdx.x; c < C; c += gridDim.y * NT) {
     float acc = 0.f;
     for (int j = 0; j < taps; ++j) {
       const int d = taps - 1 - j;          // how many rows back
@@ -91,11 +91,13 @@ extern "C" int ka_short_conv(void* out, const void* proj, int ps, int off, int C
     return (int)hipErrorInvalidValue;
   ConvArgs a{q_starts, seq_slots, positions, num_seqs, T, ps, off, C, taps, act};
   const dim3 sgrid(num_seqs, (C + NT - 1) / NT);
+  // few rows (a decode step): one channel per thread, so a thread's few dependent loads are the kernel's length
+  const dim3 cgrid(T, T >= 1024 ? 1 : (C + NT - 1) / NT);
   if (f32) {
-    short_conv_kernel<float><<<T, NT, 0, st>>>((float*)out, (const float*)proj, w, (const float*)state, a);
+    short_conv_kernel<float><<<cgrid, NT, 0, st>>>((float*)out, (const float*)proj, w, (const float*)state, a);
     if (taps > 1) short_conv_state_kernel<float><<<sgrid, NT, 0, st>>>((const float*)proj, (float*)state, a);
   } else {
-    short_conv_kernel<bf16_t><<<T, NT, 0, st>>>((bf16_t*)out, (const bf16_t*)proj, w, (const bf16_t*)state, a);
+    short_conv_kernel<bf16_t><<<cgrid, NT, 0, st>>>((bf16_t*)out, (const bf16_t*)proj, w, (const bf16_t*)state, a);
     if (taps > 1) short_conv_state_kernel<bf16_t><<<sgrid, NT, 0, st>>>((const bf16_t*)proj, (bf16_t*)state, a);
   }
   KA_CHECK_LAUNCH();

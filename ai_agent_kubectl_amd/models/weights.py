@@ -533,7 +533,8 @@ def suvapel_columns(L, rank_a: int = 0, rank_g: int = 0) -> Dict[str, int]:
     seg("g", rank_g if m.channel_decay else m.heads * m.vdim)
     if L.ff:
         seg("ff", 2 * L.ff)                                             # gate | up contiguous
-    col["total"] = o
+    # the vendor GEMM runs whole 256-column tiles fastest: a wide row block is padded with zero rows to whole tiles
+    col["total"] = (o + 1023) // 1024 * 1024 if o >= 8192 else ((o + 255) // 256 * 256 if o >= 2048 else o)
     return col
 
 

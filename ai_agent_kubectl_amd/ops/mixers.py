@@ -609,13 +609,13 @@ def sliding_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         return (_p(positions), _p(slots), _p(gate_src), gs, g_off, rows, H, G, D, Dv, int(window), int(keep_first), BS,
                 block_tables.shape[1], float(scale), _f32(q))
 
-    if (SLIDING_TILE and q_starts is not None and max_q >= 8 and q.dtype == torch.bfloat16
-            and lib.ka_sliding_attention_tile_ok(H, G, D, Dv, BS)):
+    tile = SLIDING_TILE and q.dtype == torch.bfloat16 and lib.ka_sliding_attention_tile_ok(H, G, D, Dv, BS)
+    if tile and q_starts is not None and max_q >= 8:
         # rows past the last sequence (a padded step) belong to no tile and stay zero
         out = torch.zeros((T, H * Dv), dtype=q.dtype, device=q.device)
         nd = min(int(num_decode), block_tables.shape[0])
-        if nd > 0:   # the leading one-row sequences: rows 0 .. nd - 1 only, row t is block-table row t, through the vector kernel
-            check(lib.ka_sliding_attention(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), None, nd, *tail(nd), 0,
+        if nd > 0:   # the leading one-row sequences: rows 0 .. nd - 1 only, row t is block-table row t
+            check(lib.ka_sliding_attention(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), None, nd, *tail(nd), 1,
                                            _stream()), "sliding_attention")
         if block_tables.shape[0] > nd:   # (q_starts holds absolute rows, so the remaining sequences index q and out as they are)
             check(lib.ka_sliding_attention(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables[nd:]), _p(q_starts[nd:]),
@@ -623,7 +623,8 @@ def sliding_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         return out
     out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
     check(lib.ka_sliding_attention(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(q_starts),
-                                   block_tables.shape[0], *tail(T), 0, _stream()), "sliding_attention")
+                                   block_tables.shape[0], *tail(T), 1 if tile and q_starts is None else 0, _stream()),
+          "sliding_attention")
     return out
 
 
