@@ -79,6 +79,11 @@ KA_DEV float col_sum(float v) {
     v += dpp_f<0xB1>(v);
     v += dpp_f<0x4E>(v);
     return v;
+  } else if constexpr (DPL == 8) {
+    v += dpp_f<0xB1>(v);
+    v += dpp_f<0x4E>(v);
+    v += dpp_f<0x141>(v);
+    return v;
   } else {
     return row16_sum(v);
   }
@@ -222,16 +227,37 @@ int launch_scan(float* out, const float* qk, const AT* v_src, const float* beta,
   KA_CHECK_LAUNCH();
 }
 
+// lanes per column: 0 = by the head size; 4, 8 or 16 = that many (more lanes: shorter chains per row and more
+// workgroups, at the price of staging the q / k rows once per narrower block of columns)
 template <typename AT>
 int dispatch_scan(float* out, const float* qk, const AT* v_src, const float* beta, const float* decay, float* S,
-                  const ScanArgs& a, int num_seqs, hipStream_t st) {
+                  const ScanArgs& a, int num_seqs, int lanes, hipStream_t st) {
   const int D = a.D;
-  if (D <= 16) return launch_scan<AT, 4, 4>(out, qk, v_src, beta, decay, S, a, num_seqs, st);
-  if (D <= 32) return launch_scan<AT, 8, 4>(out, qk, v_src, beta, decay, S, a, num_seqs, st);
-  if (D <= 64) return launch_scan<AT, 16, 4>(out, qk, v_src, beta, decay, S, a, num_seqs, st);
-  if (D <= 128) return launch_scan<AT, 32, 4>(out, qk, v_src, beta, decay, S, a, num_seqs, st);
-  if (D <= 256) return launch_scan<AT, 64, 4>(out, qk, v_src, beta, decay, S, a, num_seqs, st);
-  return launch_scan<AT, 32, 16>(out, qk, v_src, beta, decay, S, a, num_seqs, st);
+  // few workgroups (a step with few sequences): eight lanes a column double them and halve a row's chain
+  if (lanes == 0 && D > 32 && D <= 128 && (long)num_seqs * a.H * ((a.Dv + 63) / 64) <= 256) lanes = 8;
+#define KA_S(RPT, DPL) return launch_scan<AT, RPT, DPL>(out, qk, v_src, beta, decay, S, a, num_seqs, st)
+  if (D <= 16) KA_S(4, 4);
+  if (D <= 32) {
+    if (lanes == 8) KA_S(4, 8);
+    KA_S(8, 4);
+  }
+  if (D <= 64) {
+    if (lanes == 16) KA_S(4, 16);
+    if (lanes == 8) KA_S(8, 8);
+    KA_S(16, 4);
+  }
+  if (D <= 128) {
+    if (lanes == 16) KA_S(8, 16);
+    if (lanes == 8) KA_S(16, 8);
+    KA_S(32, 4);
+  }
+  if (D <= 256) {
+    if (lanes == 4) KA_S(64, 4);
+    if (lanes == 8) KA_S(32, 8);
+    KA_S(16, 16);
+  }
+  KA_S(32, 16);
+#undef KA_S
 }
 
 }  // namespace
@@ -255,11 +281,12 @@ extern "C" int ka_delta_prep(float* qk, float* beta, float* decay, const void* c
 // out [T, H * Dv] fp32 (rows of no sequence are left as they are)
 extern "C" int ka_delta_scan(float* out, const float* qk, const void* v_src, int vs, int v_off, const float* beta,
                              const float* decay, float* st_S, const int* seq_slots, const int* q_starts, int num_seqs,
-                             const int* positions, int H, int G, int D, int Dv, int channel, int f32, hipStream_t st) {
+                             const int* positions, int H, int G, int D, int Dv, int channel, int lanes, int f32,
+                             hipStream_t st) {
   if (num_seqs <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || D <= 0 || D > 512 || Dv <= 0 || H > 65535 || v_off < 0 || v_off + H * Dv > vs)
     return (int)hipErrorInvalidValue;
   ScanArgs a{q_starts, seq_slots, positions, vs, v_off, H, G, D, Dv, channel};
-  if (f32) return dispatch_scan<float>(out, qk, (const float*)v_src, beta, decay, st_S, a, num_seqs, st);
-  return dispatch_scan<bf16_t>(out, qk, (const bf16_t*)v_src, beta, decay, st_S, a, num_seqs, st);
+  if (f32) return dispatch_scan<float>(out, qk, (const float*)v_src, beta, decay, st_S, a, num_seqs, lanes, st);
+  return dispatch_scan<bf16_t>(out, qk, (const bf16_t*)v_src, beta, decay, st_S, a, num_seqs, lanes, st);
 }

@@ -498,7 +498,7 @@ def load_kafilorn_safetensors(path: str, cfg, device="cpu", dtype=torch.bfloat16
 #           with zero rows to a multiple of 8 columns (`suvapel_columns`): attention q | k | v | head gates,
 #           delta q | k | v | beta | decay (per head, or the low-rank pair's first half) | output gate (full, or the
 #           low-rank pair's first half), feed-forward gate | up
-#   att_conv [q + k + v channels, taps], conv [q + k + v channels, taps]                        fp32
+#   att_conv [taps, q + k + v channels], conv [taps, q + k + v channels]  (tap-major)           fp32
 #   inv_freq [rot dims / 2] fp32 (YaRN-scaled, float64 rounded once), att_wo [W, H * Dv]
 #   A_log [H], dt_bias [H] or [H * D], hnorm [H * Dv] (the shared [Dv] weight repeated per head)  fp32
 #   w_a2 [H * D, R], w_g2 [H * Dv, R] (channel decay only), wo [W, H * Dv]
@@ -562,14 +562,14 @@ def _suvapel_pack(cfg, get, device, dtype) -> Dict[str, torch.Tensor]:
             l = c + "mix.left."
             put("att_q", get(l + "q"), get(l + "k"), get(l + "v"))
             put("att_g", get(l + "g"))
-            W[p + "att_conv"] = torch.cat([get(l + "q.conv"), get(l + "k.conv"), get(l + "v.conv")])
+            W[p + "att_conv"] = torch.cat([get(l + "q.conv"), get(l + "k.conv"), get(l + "v.conv")]).t()
             W[p + "att_wo"] = get(l + "o")
             W[p + "inv_freq"] = torch.tensor(a.rot.frequencies()[0], dtype=torch.float64)
         put("q", get(r + "q"), get(r + "k"), get(r + "v"))
         put("beta", get(r + "b"))
         put("a", get(r + "a1") if m.channel_decay else get(r + "a"))
         put("g", get(r + "g1") if m.channel_decay else get(r + "g"))
-        W[p + "conv"] = torch.cat([get(r + "q.conv"), get(r + "k.conv"), get(r + "v.conv")])
+        W[p + "conv"] = torch.cat([get(r + "q.conv"), get(r + "k.conv"), get(r + "v.conv")]).t()
         W[p + "A_log"], W[p + "dt_bias"] = get(r + "A_log"), get(r + "dt_bias")
         W[p + "hnorm"] = get(r + "norm").repeat(m.heads)
         if m.channel_decay:
@@ -601,13 +601,13 @@ def suvapel_check_shapes(cfg, W: Dict[str, torch.Tensor]) -> None:
         ra = W[p + "w_a2"].shape[1] if p + "w_a2" in W else 0
         rg = W[p + "w_g2"].shape[1] if p + "w_g2" in W else 0
         want.update({p + "norm_w": (h,), p + "norm_b": (h,), p + "norm_alpha": (1,),
-                     p + "w_in": (suvapel_columns(L, ra, rg)["total"], h), p + "conv": (m.conv_channels(), m.conv),
+                     p + "w_in": (suvapel_columns(L, ra, rg)["total"], h), p + "conv": (m.conv, m.conv_channels()),
                      p + "A_log": (m.heads,), p + "dt_bias": (m.heads * m.dim if m.channel_decay else m.heads,),
                      p + "hnorm": (m.heads * m.vdim,), p + "wo": (h, m.heads * m.vdim)})
         if m.channel_decay:
             want.update({p + "w_a2": (m.heads * m.dim, ra), p + "w_g2": (m.heads * m.vdim, rg)})
         if a is not None:
-            want.update({p + "att_conv": (a.heads * a.dim + a.kv_heads * (a.dim + a.vdim), a.conv),
+            want.update({p + "att_conv": (a.conv, a.heads * a.dim + a.kv_heads * (a.dim + a.vdim)),
                          p + "att_wo": (h, a.heads * a.vdim), p + "inv_freq": (a.rot.dims // 2,)})
         if L.ff:
             want.update({p + "b_gu": (2 * L.ff,), p + "w_down": (h, L.ff), p + "b_down": (h,)})

@@ -140,7 +140,7 @@ _MIX_SIGS = {
     "ka_sliding_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, I, I, F, I, I, P],
     "ka_sliding_attention_tile_ok": [I, I, I, I, I],
     "ka_delta_prep": [P, P, P, P, I, P, I, I, P, I, I, P, P, I, I, I, I, I, I, P],
-    "ka_delta_scan": [P, P, P, I, I, P, P, P, P, P, I, P, I, I, I, I, I, I, P],
+    "ka_delta_scan": [P, P, P, I, I, P, P, P, P, P, I, P, I, I, I, I, I, I, I, P],
 }
 MIXERS_LIB = os.path.join(LIB_DIR, "libkagent_mixers.so")
 _mix: Optional[ctypes.CDLL] = None

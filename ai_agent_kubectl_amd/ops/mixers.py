@@ -530,19 +530,19 @@ def silu_mul_bias(proj: torch.Tensor, off: int, ff: int, bias: torch.Tensor) -> 
 
 def short_conv(proj: torch.Tensor, off: int, C: int, w: torch.Tensor, state: Optional[torch.Tensor],
                seq_slots: torch.Tensor, q_starts: Optional[torch.Tensor], positions: torch.Tensor, act: bool) -> torch.Tensor:
-    """A causal convolution over time per channel, y_t = sum_j w[:, j] * u_(t - taps + 1 + j), on the columns
+    """A causal convolution over time per channel, y_t = sum_j w[j] * u_(t - taps + 1 + j), on the columns
     u = proj[:, off : off + C] of each sequence's rows.  Inputs from before this step come from state[slot]
     [taps - 1, C] (the sequence's last inputs, newest last), inputs before position 0 are zero, so a slot needs no
     clearing; afterwards the state holds the last inputs including this step's.  act: silu on the result.
-    w [C, taps] fp32; state [slots, taps - 1, C] in proj's dtype (None when taps is 1).  q_starts None: row t is
-    sequence t.  -> [T, C]."""
-    taps = w.shape[1]
+    w [taps, C] fp32 (tap-major: w[j] meets the row taps - 1 - j back); state [slots, taps - 1, C] in proj's dtype
+    (None when taps is 1).  q_starts None: row t is sequence t.  -> [T, C]."""
+    taps = w.shape[0]
     if _ref(proj):
         return ref.short_conv(proj, off, C, w, state, seq_slots, q_starts, positions, act)
     lib = require_mixers()
     T, P = proj.shape
     nseq = seq_slots.shape[0]
-    assert proj.is_contiguous() and off >= 0 and off + C <= P and w.dtype == torch.float32 and w.shape == (C, taps)
+    assert proj.is_contiguous() and off >= 0 and off + C <= P and w.dtype == torch.float32 and w.shape == (taps, C)
     assert w.is_contiguous() and seq_slots.dtype == torch.int32 and positions.dtype == torch.int32 and positions.shape[0] >= T
     assert taps == 1 or (state is not None and state.dtype == proj.dtype and state.shape[1:] == (taps - 1, C)
                          and state.is_contiguous())
@@ -652,6 +652,9 @@ def delta_prep(cv: torch.Tensor, beta_src: torch.Tensor, b_off: int, a_src: torc
     return qk, beta, decay
 
 
+DELTA_LANES = 0   # lanes that hold one memory column in delta_scan: 0 = the kernel's choice by head size; 4 / 8 / 16
+
+
 def delta_scan(qk: torch.Tensor, v_src: torch.Tensor, v_off: int, beta: torch.Tensor, decay: torch.Tensor,
                st_S: torch.Tensor, seq_slots: torch.Tensor, q_starts: Optional[torch.Tensor], positions: torch.Tensor,
                H: int, G: int, D: int, Dv: int) -> torch.Tensor:
@@ -677,6 +680,6 @@ def delta_scan(qk: torch.Tensor, v_src: torch.Tensor, v_off: int, beta: torch.Te
                                                  and q_starts.shape[0] == nseq + 1)
     out = torch.zeros((T, H * Dv), dtype=torch.float32, device=qk.device)
     check(lib.ka_delta_scan(_p(out), _p(qk), _p(v_src), v_src.shape[1], v_off, _p(beta), _p(decay), _p(st_S),
-                            _p(seq_slots), _p(q_starts), nseq, _p(positions), H, G, D, Dv, int(channel), _f32(v_src),
-                            _stream()), "delta_scan")
+                            _p(seq_slots), _p(q_starts), nseq, _p(positions), H, G, D, Dv, int(channel), DELTA_LANES,
+                            _f32(v_src), _stream()), "delta_scan")
     return out

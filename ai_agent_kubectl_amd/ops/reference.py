@@ -463,11 +463,11 @@ def silu_mul_bias(proj, off: int, ff: int, bias):
 
 
 def short_conv(proj, off: int, C: int, w, state, seq_slots, q_starts, positions, act: bool):
-    """y_t = sum_j w[:, j] * u_(t - taps + 1 + j) per channel over each sequence's rows, u = proj[:, off : off + C];
+    """y_t = sum_j w[j] * u_(t - taps + 1 + j) per channel over each sequence's rows (w [taps, C]), u = proj[:, off : off + C];
     inputs before this step come from state[slot] [taps - 1, C] (the sequence's last inputs, newest last), inputs
     before position 0 are zero; the state is then advanced by the step's rows.  act: silu on the result."""
     T = proj.shape[0]
-    taps = w.shape[1]
+    taps = w.shape[0]
     out = torch.zeros((T, C), dtype=proj.dtype, device=proj.device)
     slots, pos = seq_slots.tolist(), positions.tolist()
     for i, a, b in _seq_of(T, q_starts):
@@ -480,7 +480,7 @@ def short_conv(proj, off: int, C: int, w, state, seq_slots, q_starts, positions,
             hist = hist.clone()
             hist[:taps - 1 - pos[a]] = 0.0
         full = torch.cat([hist, u])                                   # row r of the step is full[r + taps - 1]
-        y = sum(w[:, j].float() * full[j:j + (b - a)] for j in range(taps))
+        y = sum(w[j].float() * full[j:j + (b - a)] for j in range(taps))
         out[a:b] = (F.silu(y) if act else y).to(proj.dtype)
         if taps > 1:
             state[sl] = full[-(taps - 1):].to(state.dtype)

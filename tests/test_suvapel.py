@@ -182,7 +182,7 @@ def test_short_conv_whole_portions_and_decode(device, taps, C, act):
         got, at = [], 0
         for c in cuts:
             pos = torch.arange(at, at + c, dtype=torch.int32, device=device)
-            got.append(mixers.short_conv(proj[at:at + c].contiguous().to(device), off, C, w.to(device), state,
+            got.append(mixers.short_conv(proj[at:at + c].contiguous().to(device), off, C, w.t().contiguous().to(device), state,
                                          torch.tensor([1], dtype=torch.int32, device=device), _seq_meta([c], device), pos, act))
             at += c
         assert close(torch.cat(got), want)
@@ -193,7 +193,7 @@ def test_short_conv_whole_portions_and_decode(device, taps, C, act):
         rows = torch.stack([proj[t], proj[max(t - 4, 0)], proj[0]]).to(device)
         pos = torch.tensor([t, max(t - 4, 0), 0], dtype=torch.int32, device=device)
         slots = torch.tensor([2, 0 if t >= 4 else -1, -1], dtype=torch.int32, device=device)
-        o = mixers.short_conv(rows, off, C, w.to(device), state, slots, None, pos, act)
+        o = mixers.short_conv(rows, off, C, w.t().contiguous().to(device), state, slots, None, pos, act)
         outs.append(o[0])
         if t >= 4:
             assert close(o[1], want[t - 4])
@@ -216,7 +216,7 @@ def test_short_conv_unequal_sequences_in_one_step(device):
         parts = [s[lo:hi] for s in seqs]
         lens = [p.shape[0] for p in parts]
         pos = torch.cat([torch.arange(lo, lo + n) for n in lens]).to(torch.int32).to(device)
-        o = mixers.short_conv(torch.cat(parts).to(device), 0, C, w.to(device), state, slots, _seq_meta(lens, device), pos, False)
+        o = mixers.short_conv(torch.cat(parts).to(device), 0, C, w.t().contiguous().to(device), state, slots, _seq_meta(lens, device), pos, False)
         at = 0
         for i, n in enumerate(lens):
             got[i].append(o[at:at + n])
@@ -729,3 +729,50 @@ def test_mixed_steps_on_the_matrix_cores(tmp_path):
             o += len(e["tokens"])
     for k in toks:
         assert at[k] == len(toks[k]) and rel_err(np.concatenate(got[k]), want[k]) < tol("bfloat16"), k
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("lanes", [4, 8, 16])
+@pytest.mark.parametrize("H,G,D,Dv,channel", [(2, 1, 64, 70, True), (3, 3, 33, 16, False), (2, 2, 128, 40, True), (1, 1, 200, 64, False)])
+def test_delta_rule_lanes_per_column(lanes, H, G, D, Dv, channel):
+    """The kernel's forms with 4, 8 and 16 lanes per memory column give the oracle's result."""
+    from ai_agent_kubectl_amd.ops import mixers
+
+    g = torch.Generator().manual_seed(D + lanes)
+    inputs = _delta_inputs(g, 50, H, G, D, Dv, channel)
+    want = _delta_oracle(*inputs, H, G, D, Dv, channel)
+    mixers.DELTA_LANES = lanes
+    try:
+        for cuts in ([50], [20] + [1] * 30):
+            S = torch.randn(2, H, Dv, D, generator=g).cuda()
+            assert close(_delta_run("cuda", inputs, H, G, D, Dv, channel, cuts, S, 1), want, 2e-4, 2e-5), cuts
+    finally:
+        mixers.DELTA_LANES = 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("taps,act", [(4, True), (3, False), (2, True)])
+def test_short_conv_many_rows_in_bf16(taps, act):
+    """Steps of 1024 rows and more in bf16 take eight channels per thread: two sequences that continue from their
+    slots (one of them from position 1: a zero before the start), against the oracle on the same bf16 inputs."""
+    from ai_agent_kubectl_amd.ops import mixers
+
+    g = torch.Generator().manual_seed(taps)
+    C, off, lens, first = 136, 16, [700, 500], [40, 1]
+    w = torch.randn(C, taps, generator=g)
+    seqs = [torch.randn(f + n, C, generator=g).to(torch.bfloat16) for f, n in zip(first, lens)]
+    want = [oracle.short_conv(s.double().numpy(), w.double().numpy()) for s in seqs]
+    state = torch.zeros(3, taps - 1, C, dtype=torch.bfloat16).cuda()
+    slots = torch.tensor([2, 0], dtype=torch.int32).cuda()
+    wt = w.t().contiguous().cuda()
+    outs = []
+    for lo_hi in ([(0, first[0]), (0, first[1])], [(first[0], first[0] + lens[0]), (first[1], first[1] + lens[1])]):
+        parts = [s[a:b] for s, (a, b) in zip(seqs, lo_hi)]
+        rows = torch.zeros(sum(p.shape[0] for p in parts), C + 24, dtype=torch.bfloat16)
+        rows[:, off:off + C] = torch.cat(parts)
+        pos = torch.cat([torch.arange(a, b) for a, b in lo_hi]).to(torch.int32).cuda()
+        outs.append(mixers.short_conv(rows.cuda(), off, C, wt, state, slots, _seq_meta([b - a for a, b in lo_hi], "cuda"), pos, act))
+    got = outs[1].float().cpu().double().numpy()
+    ref = np.concatenate([w_[f:] for w_, f in zip(want, first)])
+    ref = oracle.silu(ref) if act else ref
+    assert np.allclose(got, ref, rtol=2e-2, atol=2e-2)
