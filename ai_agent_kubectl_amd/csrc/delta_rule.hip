@@ -103,16 +103,19 @@ __global__ __launch_bounds__(NT) void delta_scan_kernel(float* __restrict__ out,
   float* bt = vs + TB * CW;             // [TB] beta
   float* kq = bt + TB;                  // [TB] k . q
   float* gs = kq + TB;                  // [TB] (one decay per head) or [TB][Dp] (one per key channel)
-  const int seq = blockIdx.x, h = blockIdx.y;
+  // workgroups are numbered sequence by sequence, the step's last sequence first: a mixed step lists its one-row
+  // sequences first and its prompt portions last, and the long-running workgroups of the portions, dispatched first
+  // and in a row, spread evenly over the CUs (interleaved with one-row workgroups they pile up on a part of them)
+  const int H = a.H, G = a.G, D = a.D, Dv = a.Dv;
+  const int seq = gridDim.y - 1 - blockIdx.y, h = blockIdx.x % H, zb = blockIdx.x / H;
   const int slot = a.seq_slots[seq];
   if (slot < 0) return;
   const int r0 = a.q_starts ? a.q_starts[seq] : seq, r1 = a.q_starts ? a.q_starts[seq + 1] : seq + 1;
   if (r1 <= r0) return;
-  const int H = a.H, G = a.G, D = a.D, Dv = a.Dv;
   const int g = h / (H / G);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = threadIdx.x / DPL, dp = threadIdx.x % DPL;
-  const int c = blockIdx.z * CW + col;
+  const int c = zb * CW + col;
   const bool cok = c < Dv;
   float* Sp = st_S + (((size_t)slot * H + h) * Dv + (cok ? c : 0)) * D;
   const bool fresh = a.positions[r0] == 0;
@@ -141,7 +144,7 @@ __global__ __launch_bounds__(NT) void delta_scan_kernel(float* __restrict__ out,
     if (a.channel)
       for (int idx = threadIdx.x; idx < TB * Dp; idx += NT) gs[idx] = 1.f;
   }
-  const int c0 = blockIdx.z * CW;
+  const int c0 = zb * CW;
   for (int t0 = r0; t0 < r1; t0 += TB) {
     const int nt = min(TB, r1 - t0);
     __syncthreads();
@@ -222,7 +225,8 @@ int launch_scan(float* out, const float* qk, const AT* v_src, const float* beta,
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  dim3 grid(num_seqs, a.H, (a.Dv + CW - 1) / CW);
+  if (num_seqs > 65535) return (int)hipErrorInvalidValue;
+  dim3 grid(a.H * ((a.Dv + CW - 1) / CW), num_seqs);
   delta_scan_kernel<AT, RPT, DPL><<<grid, NT, lds, st>>>(out, qk, v_src, beta, decay, S, a, TB);
   KA_CHECK_LAUNCH();
 }
