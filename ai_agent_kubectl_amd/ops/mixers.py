@@ -3,9 +3,12 @@ post-norm + layer scale + residual add, PolyNorm, per-head norm + partial rotary
 attention with a chunked mask, soft-capped scores, a sink and head mixing.  `models/kafilorn.py`: residual
 streams (hyper-connections) with LayerNorm, the mLSTM gates and recurrence over state slots, latent attention
 with a sliding window and a learned sink, squared ReLU, and expert routing in groups with a choice correction.
+`models/suvapel.py`: Dynamic-Tanh norm and scaled residual sums, a gated token input, short convolutions over state
+slots, rotary positions from a frequency table, sliding-window attention that keeps the first tokens with a per-head
+gate, and the gated delta rule with a decay per head or per key channel.
 
-Dispatch follows `ops/__init__.py`: a GPU tensor goes to the HIP kernel (`csrc/norms_f32.hip`,
-`csrc/attention_chunk.hip`, built into `ops/lib/libkagent_mixers.so`) and raises if that library is
+Dispatch follows `ops/__init__.py`: a GPU tensor goes to the HIP kernel (the `csrc/*.hip` sources tagged
+`KA_HIP_LIB: mixers`, built into `ops/lib/libkagent_mixers.so`) and raises if that library is
 missing; a CPU tensor goes to the torch reference (`ops/reference.py`).  The activation dtype is bf16
 or fp32; residual, norm weights, statistics, scores and weights are fp32 in both.
 """
