@@ -14,7 +14,7 @@
 // values of one entry contiguous); slot = page * BS + offset (-1: a padding row, nothing is written or attended).
 //
 // `sliding_attention`, vector kernel: one workgroup per (token, key/value head) with the H / G query heads that
-// share it.  The visible keys (the kept first ones, then the window) are walked in page-aligned tiles of 64
+// share it (or as many of them as its accumulators hold; the rest go to further workgroups).  The visible keys (the kept first ones, then the window) are walked in page-aligned tiles of 64
 // positions with an online softmax: scores by one thread per (query head, key), the tile's maximum / sum per head by
 // one wave, weights x values by one thread per output entry, a page's values in 16-byte pieces.  Scores, weights and all sums are fp32; AT (bf16_t or float) is the type
 // of q, the cache, the gate and the output.  A decode step is the same launch with one token per sequence, so a
@@ -68,10 +68,11 @@ template <typename AT>
 __global__ __launch_bounds__(NT) void sliding_attention_kernel(AT* __restrict__ out, const AT* __restrict__ q,
                                                                const AT* __restrict__ k_cache,
                                                                const AT* __restrict__ v_cache, const AT* __restrict__ gate,
-                                                               SlideArgs a) {
+                                                               SlideArgs a, int hpw) {
   extern __shared__ float lds[];
   const int H = a.H, G = a.G, D = a.D, Dv = a.Dv, BS = a.BS;
-  const int rep = H / G;
+  // the workgroup's query heads: `hpw` of the H / G heads of key/value head g, from head g * (H / G) + hb on
+  const int hb = blockIdx.z * hpw, rep = min(hpw, H / G - hb), h0 = blockIdx.y * (H / G) + hb;
   float* qs = lds;                  // [rep * D]
   float* sc = qs + rep * D;         // [rep * KT] scores, then weights of the tile
   __shared__ float s_m[MAX_REP], s_l[MAX_REP], s_c[MAX_REP];   // running maximum, running sum, the tile's rescale
@@ -79,7 +80,7 @@ __global__ __launch_bounds__(NT) void sliding_attention_kernel(AT* __restrict__ 
   const int t = blockIdx.x, g = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int RV = rep * Dv;
-  AT* orow = out + (size_t)t * H * Dv + (size_t)g * RV;
+  AT* orow = out + ((size_t)t * H + h0) * Dv;
   if (a.slots[t] < 0 || (a.q_starts != nullptr && t >= a.q_starts[a.num_seqs])) {
     for (int i = threadIdx.x; i < RV; i += NT) stf(orow + i, 0.f);
     return;
@@ -89,7 +90,7 @@ __global__ __launch_bounds__(NT) void sliding_attention_kernel(AT* __restrict__ 
   const int* bt = a.block_tables + (size_t)seq * a.max_blocks;
   const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;   // first position of the window
   const int nk0 = min(a.keep_first, lo);                        // kept first positions that lie before the window
-  for (int i = threadIdx.x; i < rep * D; i += NT) qs[i] = ldf(q + ((size_t)t * H + (size_t)g * rep) * D + i);
+  for (int i = threadIdx.x; i < rep * D; i += NT) qs[i] = ldf(q + ((size_t)t * H + h0) * D + i);
   if (threadIdx.x < rep) {
     s_m[threadIdx.x] = -INFINITY;
     s_l[threadIdx.x] = 0.f;
@@ -191,7 +192,7 @@ __global__ __launch_bounds__(NT) void sliding_attention_kernel(AT* __restrict__ 
     if (i < RV) {
       const int r = i / Dv;
       float o = acc[u] / s_l[r];
-      if (gate != nullptr) o *= 1.0f / (1.0f + expf(-ldf(gate + (size_t)t * a.gs + a.g_off + g * rep + r)));
+      if (gate != nullptr) o *= 1.0f / (1.0f + expf(-ldf(gate + (size_t)t * a.gs + a.g_off + h0 + r)));
       stf(orow + i, o);
     }
   }
@@ -221,8 +222,8 @@ extern "C" int ka_sliding_attention(void* out, const void* q, const void* k_cach
                                     int Dv, int window, int keep_first, int BS, int max_blocks, float scale, int f32,
                                     int mode, hipStream_t st) {
   if (T <= 0) return 0;
-  if (H <= 0 || G <= 0 || H % G || H / G > MAX_REP || (H / G) * Dv > NT * MAX_ACC || D <= 0 || Dv <= 0 || BS <= 0 ||
-      window < 0 || keep_first < 0 || num_seqs <= 0)
+  if (H <= 0 || G <= 0 || H % G || Dv > NT * MAX_ACC || D <= 0 || Dv <= 0 || BS <= 0 || window < 0 || keep_first < 0 ||
+      num_seqs <= 0)
     return (int)hipErrorInvalidValue;
   if (KT % BS) return (int)hipErrorInvalidValue;   // tiles are whole pages
   if (q_starts == nullptr && T > num_seqs) return (int)hipErrorInvalidValue;   // row t reads block-table row t
@@ -232,7 +233,11 @@ extern "C" int ka_sliding_attention(void* out, const void* q, const void* k_cach
   if (!f32 && mode > 0 && (q_starts == nullptr || mode >= TILE_MIN_ROWS) && ka_sliding_attention_tile_ok(H, G, D, Dv, BS))
     return sliding_attention_tile((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                                   (const bf16_t*)gate, a, mode, T, st);
-  const int rep = H / G;
+  // query heads per workgroup: as many of a group's heads as the per-thread accumulators and the LDS hold
+  int rep = H / G;
+  rep = rep > MAX_REP ? MAX_REP : rep;
+  rep = rep * Dv > NT * MAX_ACC ? NT * MAX_ACC / Dv : rep;
+  while (rep > 1 && (size_t)(rep * D + rep * KT) * sizeof(float) > 60 * 1024) --rep;
   const size_t lds = (size_t)(rep * D + rep * KT) * sizeof(float);
   if (lds > 60 * 1024) return (int)hipErrorInvalidValue;
   if (lds > 48 * 1024) {
@@ -241,12 +246,12 @@ extern "C" int ka_sliding_attention(void* out, const void* q, const void* k_cach
     const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  const dim3 grid(T, G);
+  const dim3 grid(T, G, (H / G + rep - 1) / rep);
   if (f32)
     sliding_attention_kernel<float><<<grid, NT, lds, st>>>((float*)out, (const float*)q, (const float*)k_cache,
-                                                           (const float*)v_cache, (const float*)gate, a);
+                                                           (const float*)v_cache, (const float*)gate, a, rep);
   else
     sliding_attention_kernel<bf16_t><<<grid, NT, lds, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache,
-                                                            (const bf16_t*)v_cache, (const bf16_t*)gate, a);
+                                                            (const bf16_t*)v_cache, (const bf16_t*)gate, a, rep);
   KA_CHECK_LAUNCH();
 }

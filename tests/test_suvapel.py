@@ -285,7 +285,8 @@ def _attend(device, q, k, v, m, cuts, gate=None, dtype=torch.float32):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("H,G,D,Dv,window,keep", [(4, 2, 16, 8, 8, 2), (3, 1, 10, 7, 21, 5), (2, 2, 12, 20, 1, 0), (1, 1, 8, 8, 0, 0),
-                                                  (6, 2, 64, 128, 36, 5), (8, 1, 32, 16, 3, 9), (4, 4, 5, 3, 17, 16)])
+                                                  (6, 2, 64, 128, 36, 5), (8, 1, 32, 16, 3, 9), (4, 4, 5, 3, 17, 16),
+                                                  (20, 1, 4, 4, 5, 2), (12, 1, 16, 256, 9, 3)])
 def test_sliding_attention_windows_and_groups(device, H, G, D, Dv, window, keep):
     g = torch.Generator().manual_seed(H * 100 + D)
     T = 70
