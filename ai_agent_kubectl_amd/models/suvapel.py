@@ -57,7 +57,6 @@ class SuvapelModel:
         self.vocab_offset = 0
         self.layers: List[dict] = []
         self.cols: List[Dict[str, int]] = []
-        self.rot: List[Optional[tuple]] = []
         for i, spec in enumerate(cfg.layers):
             p = f"layers.{i}."
             L = {k[len(p):]: v for k, v in weights.items() if k.startswith(p)}
@@ -121,7 +120,7 @@ class SuvapelModel:
     def _delta(self, proj, L, m, col, li, meta: AttnMeta):
         S, cs, _ = self.state[li]
         qs = None if meta.is_decode else meta.q_starts
-        HD, GD, HV = m.heads * m.dim, m.kv_heads * m.dim, m.heads * m.vdim
+        GD = m.kv_heads * m.dim
         cv = mixers.short_conv(proj, col["q"], m.conv_channels(), L["conv"], cs, meta.state_slots, qs, meta.positions, True)
         if m.channel_decay:
             a_src, a_off = F.linear(proj[:, col["a"]:col["a"] + L["w_a2"].shape[1]], L["w_a2"]), 0
