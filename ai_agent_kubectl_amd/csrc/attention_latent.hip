@@ -6,11 +6,16 @@
 // space (q_lat = W_uk^T q, a batched GEMM outside), the attention runs multi-query over the rows with the
 // latent itself as the value, and W_uv is applied to the result (another batched GEMM outside).
 //
-//   latent_prep:   from the fused down-projection row [Q | R | Dr]: the RMS-normed query latent [Q]; the
-//                  RMS-normed c and the rotated k_r appended to the cache at the token's slot.
-//   rope_split_q:  q [T, H, D + Dr] -> the unrotated parts [H, T, D] (the batched GEMM's operand layout) and
-//                  the rotated parts [T, H, Dr] in fp32.  Rotary: entry i pairs with i + dims/2 among the
-//                  first `dims` entries, angle = position * inv_freq[i].
+//   latent_prep:   from the fused down-projection row [Q | R | Dr]: the RMS-normed query latent [Q] (Q = 0: a
+//                  model that projects its queries directly has none); the RMS-normed c and the rotated k_r
+//                  appended to the cache at the token's slot.
+//   rope_split_q:  q [T, H, D + Dr] (columns `off` .. of rows of P entries, so it may be a part of a fused
+//                  projection) -> the unrotated parts [H, T, D] (the batched GEMM's operand layout) and
+//                  the rotated parts [T, H, Dr] in fp32.  Rotary: among the first `dims` entries, entry i pairs
+//                  with i + dims/2, or (interleaved) entry 2i with 2i + 1; angle = position * inv_freq[i], cos and
+//                  sin times `mag` (a frequency table and a magnitude are what YaRN-style scalings come down to).
+//   head_gate:     o [H, T, Dv] (the batched value up-projection's result) -> [T, H * Dv], head h times
+//                  sigmoid(gate[t, h]) (gate null: the layout change only).
 //   window_attention:  s_h(j) = (q_lat_h . c_j + q_rot_h . k_r,j) * scale for the keys j with
 //                  0 <= p - j < window (window 0: all j <= p); weights exp(s) / (sum exp(s) + exp(sink_h)),
 //                  the sink optional; out_h = sum_j w_h(j) c_j, written [H, T, R].
@@ -25,10 +30,25 @@ using namespace rows;
 constexpr int KT = 64;
 constexpr int MAX_ACC = 32;   // outputs per thread: heads per workgroup * R <= NT * MAX_ACC
 
-KA_DEV float rot_entry(float self, float partner, bool first_half, float ang) {
+KA_DEV float rot_entry(float self, float partner, bool first_half, float ang, float mag) {
   float sn, cs;
   sincosf(ang, &sn, &cs);
+  sn *= mag;
+  cs *= mag;
   return first_half ? self * cs - partner * sn : self * cs + partner * sn;
+}
+
+// entry e (< dims) of a rotated vector, given the entry it is paired with (rot_partner)
+KA_DEV float rot_at(float self, float partner, int e, int dims, bool interleaved, float pos, const float* inv_freq,
+                    float mag) {
+  const int half = dims >> 1;
+  const bool first = interleaved ? (e & 1) == 0 : e < half;
+  const int j = interleaved ? e >> 1 : (e < half ? e : e - half);
+  return rot_entry(self, partner, first, pos * inv_freq[j], mag);
+}
+KA_DEV int rot_partner(int e, int dims, bool interleaved) {
+  const int half = dims >> 1;
+  return interleaved ? e ^ 1 : (e < half ? e + half : e - half);
 }
 
 template <typename AT>
@@ -36,17 +56,20 @@ __global__ __launch_bounds__(NT) void latent_prep_kernel(AT* __restrict__ cq, co
                                                          int R, int Dr, const float* __restrict__ w_q,
                                                          const float* __restrict__ w_kv, const float* __restrict__ inv_freq,
                                                          const int* __restrict__ positions, const int* __restrict__ slots,
-                                                         AT* __restrict__ cache, int rot_dims, float eps) {
+                                                         AT* __restrict__ cache, int rot_dims, float eps,
+                                                         int interleaved, float mag) {
   __shared__ float red[NW];
   const int t = blockIdx.x;
   const AT* row = proj + (size_t)t * P;
-  float s = 0.f;
-  for (int i = threadIdx.x; i < Q; i += NT) {
-    const float v = ldf(row + i);
-    s += v * v;
+  float s = 0.f, inv;
+  if (Q > 0) {
+    for (int i = threadIdx.x; i < Q; i += NT) {
+      const float v = ldf(row + i);
+      s += v * v;
+    }
+    inv = 1.0f / sqrtf(block_sum(s, red) / (float)Q + eps);
+    for (int i = threadIdx.x; i < Q; i += NT) stf(cq + (size_t)t * Q + i, ldf(row + i) * inv * w_q[i]);
   }
-  float inv = 1.0f / sqrtf(block_sum(s, red) / (float)Q + eps);
-  for (int i = threadIdx.x; i < Q; i += NT) stf(cq + (size_t)t * Q + i, ldf(row + i) * inv * w_q[i]);
   if (cache == nullptr) return;
   const int slot = slots[t];
   if (slot < 0) return;
@@ -58,14 +81,13 @@ __global__ __launch_bounds__(NT) void latent_prep_kernel(AT* __restrict__ cq, co
   inv = 1.0f / sqrtf(block_sum(s, red) / (float)R + eps);
   AT* dst = cache + (size_t)slot * (R + Dr);
   for (int i = threadIdx.x; i < R; i += NT) stf(dst + i, ldf(row + Q + i) * inv * w_kv[i]);
-  const int half = rot_dims >> 1;
   const float pos = (float)positions[t];
   const AT* kr = row + Q + R;
   for (int i = threadIdx.x; i < Dr; i += NT) {
     float o = ldf(kr + i);
     if (i < rot_dims) {
-      const int j = i < half ? i : i - half;
-      o = rot_entry(o, ldf(kr + (i < half ? i + half : i - half)), i < half, pos * inv_freq[j]);
+      const float pr = ldf(kr + rot_partner(i, rot_dims, interleaved));
+      o = rot_at(o, pr, i, rot_dims, interleaved, pos, inv_freq, mag);
     }
     stf(dst + R + i, o);
   }
@@ -73,13 +95,14 @@ __global__ __launch_bounds__(NT) void latent_prep_kernel(AT* __restrict__ cq, co
 
 template <typename AT>
 __global__ __launch_bounds__(NT) void rope_split_q_kernel(AT* __restrict__ qn, float* __restrict__ qr,
-                                                          const AT* __restrict__ q, const float* __restrict__ inv_freq,
+                                                          const AT* __restrict__ q, int P, int off,
+                                                          const float* __restrict__ inv_freq,
                                                           const int* __restrict__ positions, int T, int H, int D, int Dr,
-                                                          int rot_dims) {
+                                                          int rot_dims, int interleaved, float mag) {
   const int t = blockIdx.x;
-  const int half = rot_dims >> 1, DD = D + Dr;
+  const int DD = D + Dr;
   const float pos = (float)positions[t];
-  const AT* row = q + (size_t)t * H * DD;
+  const AT* row = q + (size_t)t * P + off;
   for (int idx = threadIdx.x; idx < H * DD; idx += NT) {
     const int h = idx / DD, i = idx % DD;
     if (i < D) {
@@ -88,11 +111,24 @@ __global__ __launch_bounds__(NT) void rope_split_q_kernel(AT* __restrict__ qn, f
       const int e = i - D;
       float o = ldf(row + idx);
       if (e < rot_dims) {
-        const int j = e < half ? e : e - half;
-        o = rot_entry(o, ldf(row + h * DD + D + (e < half ? e + half : e - half)), e < half, pos * inv_freq[j]);
+        const float pr = ldf(row + h * DD + D + rot_partner(e, rot_dims, interleaved));
+        o = rot_at(o, pr, e, rot_dims, interleaved, pos, inv_freq, mag);
       }
       qr[((size_t)t * H + h) * Dr + e] = o;
     }
+  }
+}
+
+template <typename AT>
+__global__ __launch_bounds__(NT) void head_gate_kernel(AT* __restrict__ out, const AT* __restrict__ o,
+                                                       const AT* __restrict__ gate, int gs, int g_off, int T, int H,
+                                                       int Dv) {
+  const int t = blockIdx.x;
+  for (int idx = threadIdx.x; idx < H * Dv; idx += NT) {
+    const int h = idx / Dv, d = idx - h * Dv;
+    float v = ldf(o + ((size_t)h * T + t) * Dv + d);
+    if (gate != nullptr) v *= 1.0f / (1.0f + expf(-ldf(gate + (size_t)t * gs + g_off + h)));
+    stf(out + (size_t)t * H * Dv + idx, v);
   }
 }
 
@@ -445,25 +481,39 @@ int launch_tile(bf16_t* out, const bf16_t* q_lat, const float* q_rot, const bf16
 
 extern "C" int ka_latent_prep(void* cq, const void* proj, int T, int P, int Q, int R, int Dr, const float* w_q,
                               const float* w_kv, const float* inv_freq, const int* positions, const int* slots,
-                              void* cache, int rot_dims, float eps, int f32, hipStream_t st) {
+                              void* cache, int rot_dims, float eps, int interleaved, float mag, int f32, hipStream_t st) {
   if (T <= 0) return 0;
-  if (Q <= 0 || P < Q || (cache != nullptr && (P < Q + R + Dr || R <= 0)) || rot_dims < 0 || rot_dims > Dr || (rot_dims & 1))
+  if (Q < 0 || P < Q || (Q == 0 && cache == nullptr) || (cache != nullptr && (P < Q + R + Dr || R <= 0)) || rot_dims < 0 || rot_dims > Dr || (rot_dims & 1))
     return (int)hipErrorInvalidValue;
   if (f32)
     latent_prep_kernel<float><<<T, NT, 0, st>>>((float*)cq, (const float*)proj, P, Q, R, Dr, w_q, w_kv, inv_freq, positions,
-                                                slots, (float*)cache, rot_dims, eps);
+                                                slots, (float*)cache, rot_dims, eps, interleaved, mag);
   else
     latent_prep_kernel<bf16_t><<<T, NT, 0, st>>>((bf16_t*)cq, (const bf16_t*)proj, P, Q, R, Dr, w_q, w_kv, inv_freq,
-                                                 positions, slots, (bf16_t*)cache, rot_dims, eps);
+                                                 positions, slots, (bf16_t*)cache, rot_dims, eps, interleaved, mag);
   KA_CHECK_LAUNCH();
 }
 
-extern "C" int ka_rope_split_q(void* qn, float* qr, const void* q, const float* inv_freq, const int* positions, int T,
-                               int H, int D, int Dr, int rot_dims, int f32, hipStream_t st) {
+extern "C" int ka_rope_split_q(void* qn, float* qr, const void* q, int P, int off, const float* inv_freq,
+                               const int* positions, int T, int H, int D, int Dr, int rot_dims, int interleaved, float mag,
+                               int f32, hipStream_t st) {
   if (T <= 0) return 0;
-  if (rot_dims < 0 || rot_dims > Dr || (rot_dims & 1)) return (int)hipErrorInvalidValue;
-  if (f32) rope_split_q_kernel<float><<<T, NT, 0, st>>>((float*)qn, qr, (const float*)q, inv_freq, positions, T, H, D, Dr, rot_dims);
-  else rope_split_q_kernel<bf16_t><<<T, NT, 0, st>>>((bf16_t*)qn, qr, (const bf16_t*)q, inv_freq, positions, T, H, D, Dr, rot_dims);
+  if (rot_dims < 0 || rot_dims > Dr || (rot_dims & 1) || off < 0 || off + H * (D + Dr) > P) return (int)hipErrorInvalidValue;
+  if (f32)
+    rope_split_q_kernel<float><<<T, NT, 0, st>>>((float*)qn, qr, (const float*)q, P, off, inv_freq, positions, T, H, D, Dr,
+                                                 rot_dims, interleaved, mag);
+  else
+    rope_split_q_kernel<bf16_t><<<T, NT, 0, st>>>((bf16_t*)qn, qr, (const bf16_t*)q, P, off, inv_freq, positions, T, H, D, Dr,
+                                                  rot_dims, interleaved, mag);
+  KA_CHECK_LAUNCH();
+}
+
+extern "C" int ka_head_gate(void* out, const void* o, const void* gate, int gs, int g_off, int T, int H, int Dv, int f32,
+                            hipStream_t st) {
+  if (T <= 0) return 0;
+  if (H <= 0 || Dv <= 0 || (gate != nullptr && (g_off < 0 || g_off + H > gs))) return (int)hipErrorInvalidValue;
+  if (f32) head_gate_kernel<float><<<T, NT, 0, st>>>((float*)out, (const float*)o, (const float*)gate, gs, g_off, T, H, Dv);
+  else head_gate_kernel<bf16_t><<<T, NT, 0, st>>>((bf16_t*)out, (const bf16_t*)o, (const bf16_t*)gate, gs, g_off, T, H, Dv);
   KA_CHECK_LAUNCH();
 }
 

@@ -14,7 +14,14 @@ struct SlideArgs {
   int num_seqs, H, G, D, Dv, window, keep_first, BS, max_blocks;
   int gs, g_off;             // gate row stride and column offset
   float scale;
+  const float* dist;         // [3, H] or null.  Set: no softmax; a visible key's weight is
+                             // sigmoid(score - dist[0][h] * log(1 + dist[1][h] * (p - j)) + dist[2][h]), not normalised
 };
+
+// the unnormalised weight of the key at distance `d` behind the query (SlideArgs::dist of head h in r1, r2, pb)
+KA_DEV float dist_sigmoid(float score, float r1, float r2, float pb, int d) {
+  return 1.0f / (1.0f + expf(-(score - r1 * log1pf(r2 * (float)d) + pb)));
+}
 
 // the matrix-core kernel (bf16): 1 if it takes the shape
 extern "C" int ka_sliding_attention_tile_ok(int H, int G, int D, int Dv, int BS);

@@ -6,8 +6,13 @@
 //   visible(p, j) = j <= p and (p - j < window or j < keep_first)      (window 0: every j <= p)
 //   a kept key is rotated and masked by the position it was written at, like any other key;
 //   head h's result is multiplied by sigmoid(gate[t, h]), one number per token and head (gate null: none).
+//   With `dist` (three numbers r1, r2, pb per head) there is no softmax: the weight of a visible key is
+//   sigmoid(score - r1 log(1 + r2 (p - j)) + pb), a logarithmic distance bias taken off the score, and the
+//   weights are summed against the values as they are.
 //
-// `rope_append`: rows [q (H x D) | k (G x D) | v (G x Dv)] -> q [T, H, D], rotary positions on the first `rot`
+// `rope_append`: rows [q (H x D) | k (G x D) | v (G x Dv)] -> q [T, H, D]; with q_norm / k_norm [D] every q / k
+// head is first divided by its root mean square (eps inside the root) and multiplied by that weight (one workgroup
+// per token, a wave per head); rotary positions on the first `rot`
 // entries of every q and k head (pairs (i, i + rot/2), angle = position * inv_freq[i] in fp32, cos and sin times
 // `mag`: a frequency table and a magnitude are what YaRN-style scalings come down to); the rotated keys and the
 // values go to the paged cache.  Cache layout: k_cache [NB, G, BS, D] (token-major), v_cache [NB, G, Dv, BS] (a page's
@@ -34,20 +39,40 @@ __global__ __launch_bounds__(NT) void rope_append_kernel(AT* __restrict__ q_out,
                                                          const float* __restrict__ inv_freq, float mag,
                                                          const int* __restrict__ positions, const int* __restrict__ slots,
                                                          AT* __restrict__ k_cache, AT* __restrict__ v_cache, int H, int G,
-                                                         int D, int Dv, int rot, int BS) {
+                                                         int D, int Dv, int rot, int BS, const float* __restrict__ q_norm,
+                                                         const float* __restrict__ k_norm, float eps) {
+  extern __shared__ float hinv[];   // [H + G] 1 / rms of each q and k head (only with a norm)
   const int t = blockIdx.x;
   const int half = rot >> 1;
   const float pos = (float)positions[t];
   const int slot = slots[t];
   const AT* row = qkv + (size_t)t * ((H + G) * D + G * Dv);
   const size_t page = slot >= 0 ? (size_t)(slot / BS) : 0, offs = slot >= 0 ? (size_t)(slot % BS) : 0;
+  const bool normed = q_norm != nullptr || k_norm != nullptr;
+  if (normed) {
+    const int lane = threadIdx.x & 63;
+    for (int hh = threadIdx.x >> 6; hh < H + G; hh += NW) {
+      float s = 0.f;
+      for (int i = lane; i < D; i += 64) {
+        const float v = ldf(row + hh * D + i);
+        s += v * v;
+      }
+      s = wave_sum(s);
+      if (lane == 0) hinv[hh] = (hh < H ? q_norm : k_norm) != nullptr ? 1.0f / sqrtf(s / (float)D + eps) : 1.0f;
+    }
+    __syncthreads();
+  }
   for (int idx = threadIdx.x; idx < (H + G) * D; idx += NT) {
     const int hh = idx / D, i = idx % D;
     if (hh >= H && slot < 0) break;
     float o = ldf(row + idx);
+    const float* nw = hh < H ? q_norm : k_norm;
+    if (nw != nullptr) o *= hinv[hh] * nw[i];
     if (i < rot) {
       const int j = i < half ? i : i - half;
-      const float partner = ldf(row + (i < half ? idx + half : idx - half));
+      const int pi = i < half ? i + half : i - half;
+      float partner = ldf(row + hh * D + pi);
+      if (nw != nullptr) partner *= hinv[hh] * nw[pi];
       float sn, cs;
       sincosf(pos * inv_freq[j], &sn, &cs);
       sn *= mag;
@@ -91,9 +116,11 @@ __global__ __launch_bounds__(NT) void sliding_attention_kernel(AT* __restrict__ 
   const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;   // first position of the window
   const int nk0 = min(a.keep_first, lo);                        // kept first positions that lie before the window
   for (int i = threadIdx.x; i < rep * D; i += NT) qs[i] = ldf(q + ((size_t)t * H + h0) * D + i);
-  if (threadIdx.x < rep) {
+  const bool sig = a.dist != nullptr;
+  if (threadIdx.x < rep) {   // sigmoid weights are final as they are: no maximum, no rescale, no denominator
     s_m[threadIdx.x] = -INFINITY;
-    s_l[threadIdx.x] = 0.f;
+    s_l[threadIdx.x] = sig ? 1.f : 0.f;
+    s_c[threadIdx.x] = 1.f;
   }
   float acc[MAX_ACC];
 #pragma unroll
@@ -137,11 +164,14 @@ __global__ __launch_bounds__(NT) void sliding_attention_kernel(AT* __restrict__ 
             }
           }
           s *= a.scale;
+          if (sig) s = dist_sigmoid(s, a.dist[h0 + r], a.dist[H + h0 + r], a.dist[2 * H + h0 + r], p - pos);
+        } else if (sig) {
+          s = 0.f;
         }
         sc[it] = s;
       }
       __syncthreads();
-      for (int r = wave; r < rep; r += NW) {      // the tile's place in head r's running softmax
+      for (int r = wave; r < rep && !sig; r += NW) {      // the tile's place in head r's running softmax
         const float s = sc[r * KT + lane];
         const float mo = s_m[r];
         const float m = fmaxf(mo, wave_max(s));   // finite: a tile holds at least one position of its span
@@ -202,16 +232,19 @@ __global__ __launch_bounds__(NT) void sliding_attention_kernel(AT* __restrict__ 
 
 extern "C" int ka_rope_append(void* q_out, const void* qkv, const float* inv_freq, float mag, const int* positions,
                               const int* slots, void* k_cache, void* v_cache, int T, int H, int G, int D, int Dv, int rot,
-                              int BS, int f32, hipStream_t st) {
+                              int BS, const float* q_norm, const float* k_norm, float eps, int f32, hipStream_t st) {
   if (T <= 0) return 0;
   if (D <= 0 || Dv <= 0 || rot < 0 || rot > D || (rot & 1) || BS <= 0 || H <= 0 || G <= 0 || (rot > 0 && inv_freq == nullptr))
     return (int)hipErrorInvalidValue;
+  const size_t lds = (size_t)(H + G) * sizeof(float);
+  if (lds > 32 * 1024) return (int)hipErrorInvalidValue;
   if (f32)
-    rope_append_kernel<float><<<T, NT, 0, st>>>((float*)q_out, (const float*)qkv, inv_freq, mag, positions, slots,
-                                                (float*)k_cache, (float*)v_cache, H, G, D, Dv, rot, BS);
+    rope_append_kernel<float><<<T, NT, lds, st>>>((float*)q_out, (const float*)qkv, inv_freq, mag, positions, slots,
+                                                  (float*)k_cache, (float*)v_cache, H, G, D, Dv, rot, BS, q_norm, k_norm, eps);
   else
-    rope_append_kernel<bf16_t><<<T, NT, 0, st>>>((bf16_t*)q_out, (const bf16_t*)qkv, inv_freq, mag, positions, slots,
-                                                 (bf16_t*)k_cache, (bf16_t*)v_cache, H, G, D, Dv, rot, BS);
+    rope_append_kernel<bf16_t><<<T, NT, lds, st>>>((bf16_t*)q_out, (const bf16_t*)qkv, inv_freq, mag, positions, slots,
+                                                   (bf16_t*)k_cache, (bf16_t*)v_cache, H, G, D, Dv, rot, BS, q_norm, k_norm,
+                                                   eps);
   KA_CHECK_LAUNCH();
 }
 
@@ -219,15 +252,15 @@ extern "C" int ka_rope_append(void* q_out, const void* qkv, const float* inv_fre
 extern "C" int ka_sliding_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
                                     const int* block_tables, const int* q_starts, int num_seqs, const int* positions,
                                     const int* slots, const void* gate, int gs, int g_off, int T, int H, int G, int D,
-                                    int Dv, int window, int keep_first, int BS, int max_blocks, float scale, int f32,
-                                    int mode, hipStream_t st) {
+                                    int Dv, int window, int keep_first, int BS, int max_blocks, float scale,
+                                    const float* dist, int f32, int mode, hipStream_t st) {
   if (T <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || Dv > NT * MAX_ACC || D <= 0 || Dv <= 0 || BS <= 0 || window < 0 || keep_first < 0 ||
       num_seqs <= 0)
     return (int)hipErrorInvalidValue;
   if (KT % BS) return (int)hipErrorInvalidValue;   // tiles are whole pages
   if (q_starts == nullptr && T > num_seqs) return (int)hipErrorInvalidValue;   // row t reads block-table row t
-  SlideArgs a{block_tables, q_starts, positions, slots, num_seqs, H, G, D, Dv, window, keep_first, BS, max_blocks, gs, g_off, scale};
+  SlideArgs a{block_tables, q_starts, positions, slots, num_seqs, H, G, D, Dv, window, keep_first, BS, max_blocks, gs, g_off, scale, dist};
   // bf16 on the matrix cores where the shape allows: prompt portions (mode = the longest run of rows of one
   // sequence in the step) and single rows (q_starts null); mode 0 asks for the vector kernel
   if (!f32 && mode > 0 && (q_starts == nullptr || mode >= TILE_MIN_ROWS) && ka_sliding_attention_tile_ok(H, G, D, Dv, BS))

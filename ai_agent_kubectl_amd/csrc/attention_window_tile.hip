@@ -17,6 +17,8 @@
 // No LDS, no barrier.  The rescale factors and the final 1 / sum * sigmoid(gate) reach the accumulator rows (queries
 // 4 (lane >> 4) + r) by lane reads.  Slots of the last page beyond the rows' positions may hold another sequence's
 // old values: their weights are zero and their value bits are cleared before the product.
+// SIG (SlideArgs::dist set): the weights are sigmoids of the biased scores and final as they are, so the maximum, the
+// rescale and the denominator fall away and the waves' partial results of a single row are simply added.
 #include "attention_window.h"
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -40,7 +42,7 @@ KA_DEV void split2(const f32x4& p, s16x4& hi, s16x4& lo) {
 // DEC true: single rows (a decode step, or the one-row sequences of a mixed step).  The query columns are the H / G
 //   heads of the key/value group for ONE row, so a page is read once for all of them; the workgroup's four waves
 //   take every fourth step of the pages with a softmax of their own and are merged through LDS at the end.
-template <int DK, int DB, bool DEC>   // D = 32 DK, Dv = 16 DB
+template <int DK, int DB, bool DEC, bool SIG>   // D = 32 DK, Dv = 16 DB
 __global__ __launch_bounds__(512) void sliding_tile_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
                                                            const bf16_t* __restrict__ k_cache,
                                                            const bf16_t* __restrict__ v_cache,
@@ -75,6 +77,12 @@ __global__ __launch_bounds__(512) void sliding_tile_kernel(bf16_t* __restrict__ 
   const int p_q = DEC ? P0 : P0 + col;             // this lane's query position
   const int row_q = DEC ? r0 : r0 + cq;            // its row of q / gate / out
   const int h_q = g * rep + (DEC ? cq : wave);     // its query head
+  float r1 = 0.f, r2 = 0.f, pb = 0.f;              // the lane's head's distance bias and score offset
+  if constexpr (SIG) {
+    r1 = a.dist[h_q];
+    r2 = a.dist[H + h_q];
+    pb = a.dist[2 * H + h_q];
+  }
   bf16x8 qf[DK];
   {
     const bf16_t* qp = q + ((size_t)row_q * H + h_q) * D + 8 * grp;
@@ -112,11 +120,19 @@ __global__ __launch_bounds__(512) void sliding_tile_kernel(bf16_t* __restrict__ 
         for (int r = 0; r < 4; ++r) {
           const int j = pg * PG + 4 * grp + r;
           const bool ok = valid_q && j <= p_q && (p_q - j < W || j < a.keep_first);
-          sv[u][r] = ok ? s[r] * a.scale : -INFINITY;
-          mt = fmaxf(mt, sv[u][r]);
+          if constexpr (SIG) {
+            const float z = s[r] * a.scale - r1 * __logf(1.0f + r2 * (float)(p_q - j)) + pb;
+            sv[u][r] = ok ? 1.0f / (1.0f + __expf(-z)) : 0.f;
+          } else {
+            sv[u][r] = ok ? s[r] * a.scale : -INFINITY;
+            mt = fmaxf(mt, sv[u][r]);
+          }
         }
+      } else if constexpr (SIG) {
+        sv[u] = f32x4{0.f, 0.f, 0.f, 0.f};
       }
     }
+    if constexpr (!SIG) {
     mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
     mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
     const float m_new = fmaxf(m_run, mt);
@@ -142,6 +158,7 @@ __global__ __launch_bounds__(512) void sliding_tile_kernel(bf16_t* __restrict__ 
 #pragma unroll
         for (int r = 0; r < 4; ++r) O[db][r] *= cr[r];
     }
+    }   // !SIG
 #pragma unroll
     for (int u = 0; u < NP; ++u) {
       if (i0 + u < total) {
@@ -170,9 +187,9 @@ __global__ __launch_bounds__(512) void sliding_tile_kernel(bf16_t* __restrict__ 
     float* sm = lds;                     // [nw][rep]
     float* sl = sm + nw * rep;           // [nw][rep]
     float* so = sl + nw * rep;           // [nw][rep][Dv]
-    if (grp == 0 && col < rep) {
-      sm[wave * rep + col] = m_run;
-      sl[wave * rep + col] = l_run;
+    if (grp == 0 && col < rep) {   // SIG: equal maxima and denominators 1 / nw make the merge below a plain sum
+      sm[wave * rep + col] = SIG ? 0.f : m_run;
+      sl[wave * rep + col] = SIG ? 1.0f / (float)nw : l_run;
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -199,7 +216,7 @@ __global__ __launch_bounds__(512) void sliding_tile_kernel(bf16_t* __restrict__ 
       out[((size_t)r0 * H + g * rep + hq) * Dv + d] = f2bf(o);
     }
   } else {
-    float fin = valid_q ? 1.0f / l_run : 0.f;
+    float fin = valid_q ? (SIG ? 1.0f : 1.0f / l_run) : 0.f;
     if (gate != nullptr && valid_q) fin *= 1.0f / (1.0f + __expf(-bf2f(gate[(size_t)row_q * a.gs + a.g_off + h_q])));
     float fr[4];
 #pragma unroll
@@ -218,7 +235,7 @@ __global__ __launch_bounds__(512) void sliding_tile_kernel(bf16_t* __restrict__ 
 
 constexpr int DEC_WAVES = 4;
 
-template <int DK, int DB>
+template <int DK, int DB, bool SIG>
 int launch_tile(bf16_t* out, const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const bf16_t* gate,
                 const SlideArgs& a, int max_q, int rows_, hipStream_t st) {
   if (a.q_starts == nullptr) {   // single rows
@@ -226,14 +243,14 @@ int launch_tile(bf16_t* out, const bf16_t* q, const bf16_t* k_cache, const bf16_
     const size_t lds = (size_t)(DEC_WAVES * rep * (2 + 16 * DB)) * sizeof(float);
     if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
     if (lds > 48 * 1024) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(sliding_tile_kernel<DK, DB, true>),
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(sliding_tile_kernel<DK, DB, true, SIG>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       if (e != hipSuccess) return (int)e;
     }
-    sliding_tile_kernel<DK, DB, true><<<dim3(rows_, a.G), 64 * DEC_WAVES, lds, st>>>(out, q, k_cache, v_cache, gate, a, 1);
+    sliding_tile_kernel<DK, DB, true, SIG><<<dim3(rows_, a.G), 64 * DEC_WAVES, lds, st>>>(out, q, k_cache, v_cache, gate, a, 1);
   } else {
     const int tiles = (max_q + 15) / 16;
-    sliding_tile_kernel<DK, DB, false><<<dim3(a.num_seqs * tiles, a.G), 64 * (a.H / a.G), 0, st>>>(out, q, k_cache, v_cache,
+    sliding_tile_kernel<DK, DB, false, SIG><<<dim3(a.num_seqs * tiles, a.G), 64 * (a.H / a.G), 0, st>>>(out, q, k_cache, v_cache,
                                                                                                  gate, a, tiles);
   }
   KA_CHECK_LAUNCH();
@@ -252,7 +269,9 @@ int sliding_attention_tile(bf16_t* out, const bf16_t* q, const bf16_t* k_cache, 
                            const SlideArgs& a, int max_q, int rows_, hipStream_t st) {
   if (!ka_sliding_attention_tile_ok(a.H, a.G, a.D, a.Dv, a.BS) || (a.q_starts != nullptr ? max_q <= 0 : rows_ <= 0))
     return (int)hipErrorInvalidValue;
-#define KA_T(DK, DB) return launch_tile<DK, DB>(out, q, k_cache, v_cache, gate, a, max_q, rows_, st)
+#define KA_T(DK, DB)                                                                                        \
+  return a.dist != nullptr ? launch_tile<DK, DB, true>(out, q, k_cache, v_cache, gate, a, max_q, rows_, st) \
+                           : launch_tile<DK, DB, false>(out, q, k_cache, v_cache, gate, a, max_q, rows_, st)
   if (a.D == 64) {
     if (a.Dv == 64) KA_T(2, 4);
     if (a.Dv == 128) KA_T(2, 8);

@@ -4,14 +4,18 @@
 // (models/kafilorn.py).
 //
 //   moe_route:  z = W_router h in fp32 (weights [E, W] fp32, one wave per logit); s = softmax(z) over all
-//               experts; choice = s + correction (optional).  The experts form `groups` equal groups of
+//               experts, or (sigmoid) s = sigmoid(z) per expert; choice = s + correction (optional).  The experts form `groups` equal groups of
 //               neighbours; a group's score is its largest choice; only experts of the `keep` best groups
 //               can be chosen.  The `top` largest choices are taken (ties: the lower index); the weights
-//               are their s (without the correction) over their sum (+ 1e-20).  One workgroup per token.
+//               are their s (without the correction) over their sum (+ 1e-20), or (renorm 0) their s as they
+//               are.  One workgroup per token.
 //   moe_gate_up / moe_down:  for step sizes of a few rows (decode), the chosen experts as matrix-vector
 //               products straight from the stacked expert weights, no routing lists and no host read, so a
 //               decode step can be captured: act[t, k] = silu(gate_e h) * (up_e h) with e = ids[t, k], then
 //               out[t] = sum_k w[t, k] down_e act[t, k] in fp32.  Any dtype; the fp32 engine's path.
+//               in_scale: the weight multiplies the expert's INPUT instead of its output; as the two projections
+//               are linear it is applied to their fp32 results, act = silu(w gate_e h) * (w up_e h), and the
+//               outputs are summed as they are.
 //   moe_grouped:  the same step in bf16 on the matrix cores, rows grouped by expert (below).
 #include "rows_f32.h"
 
@@ -25,7 +29,7 @@ template <typename AT>
 __global__ __launch_bounds__(NT) void moe_route_kernel(int* __restrict__ ids, float* __restrict__ wts,
                                                        const AT* __restrict__ h, const float* __restrict__ wr,
                                                        const float* __restrict__ correction, int width, int E, int top,
-                                                       int groups, int keep) {
+                                                       int groups, int keep, int sigmoid, int renorm) {
   __shared__ float z[MAX_E];      // logits, then scores
   __shared__ float ch[MAX_E];     // choice scores (minus infinity once taken or outside the kept groups)
   __shared__ float gs[MAX_E];     // group scores
@@ -58,14 +62,16 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(int* __restrict__ ids, fl
   }
   __syncthreads();
   if (wave != 0) return;
-  float mx = -INFINITY;
-  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
-  mx = wave_max(mx);
-  float sum = 0.f;
-  for (int e = lane; e < E; e += 64) sum += expf(z[e] - mx);
-  sum = wave_sum(sum);
+  float mx = -INFINITY, sum = 1.f;
+  if (!sigmoid) {
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    mx = wave_max(mx);
+    sum = 0.f;
+    for (int e = lane; e < E; e += 64) sum += expf(z[e] - mx);
+    sum = wave_sum(sum);
+  }
   for (int e = lane; e < E; e += 64) {
-    const float s = expf(z[e] - mx) / sum;
+    const float s = sigmoid ? 1.0f / (1.0f + expf(-z[e])) : expf(z[e] - mx) / sum;
     z[e] = s;
     ch[e] = s + (correction != nullptr ? correction[e] : 0.f);
   }
@@ -109,7 +115,7 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(int* __restrict__ ids, fl
   }
   if (lane < top) {
     ids[(size_t)t * top + lane] = mid;
-    wts[(size_t)t * top + lane] = mine / (wsum + 1e-20f);
+    wts[(size_t)t * top + lane] = renorm ? mine / (wsum + 1e-20f) : mine;
   }
 }
 
@@ -118,10 +124,11 @@ constexpr int FPW = 4;   // outputs per wave
 template <typename AT>
 __global__ __launch_bounds__(NT) void moe_gate_up_kernel(AT* __restrict__ act, const AT* __restrict__ h,
                                                          const AT* __restrict__ w_gu, const int* __restrict__ ids,
-                                                         int width, int ff, int top) {
+                                                         const float* __restrict__ in_w, int width, int ff, int top) {
   extern __shared__ float hs[];   // [width]
   const int row = blockIdx.x, t = row / top;
   const int e = ids[row];
+  const float isc = in_w != nullptr ? in_w[row] : 1.f;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int i = threadIdx.x; i < width; i += NT) hs[i] = ldf(h + (size_t)t * width + i);
   __syncthreads();
@@ -136,8 +143,8 @@ __global__ __launch_bounds__(NT) void moe_gate_up_kernel(AT* __restrict__ act, c
       sg += hs[i] * ldf(g + i);
       su += hs[i] * ldf(up + i);
     }
-    sg = wave_sum(sg);
-    su = wave_sum(su);
+    sg = wave_sum(sg) * isc;
+    su = wave_sum(su) * isc;
     if (lane == 0) stf(act + (size_t)row * ff + f, sg / (1.f + expf(-sg)) * su);
   }
 }
@@ -147,6 +154,7 @@ template <typename AT>
 __global__ __launch_bounds__(NT) void moe_down_kernel(float* __restrict__ out, const AT* __restrict__ act,
                                                       const AT* __restrict__ w_down, const int* __restrict__ ids,
                                                       const float* __restrict__ wts, int width, int ff, int top) {
+  // wts null: the rows are summed as they are
   extern __shared__ float as[];   // [top][ff]
   __shared__ int se[MAX_TOP];
   __shared__ float sw[MAX_TOP];
@@ -155,7 +163,7 @@ __global__ __launch_bounds__(NT) void moe_down_kernel(float* __restrict__ out, c
   for (int i = threadIdx.x; i < top * ff; i += NT) as[i] = ldf(act + (size_t)t * top * ff + i);
   if (threadIdx.x < top) {
     se[threadIdx.x] = ids[(size_t)t * top + threadIdx.x];
-    sw[threadIdx.x] = wts[(size_t)t * top + threadIdx.x];
+    sw[threadIdx.x] = wts != nullptr ? wts[(size_t)t * top + threadIdx.x] : 1.f;
   }
   __syncthreads();
   for (int u = 0; u < FPW; ++u) {
@@ -178,7 +186,8 @@ __global__ __launch_bounds__(NT) void moe_down_kernel(float* __restrict__ out, c
 // are read once.  A workgroup takes (expert e, 64 output features): it lists the (token, choice) rows routed to e
 // and runs them, 16 at a time, as the M rows of MFMA 16x16x32 products against the expert's weight rows (B
 // fragments are 16-byte loads straight from the stacked weights, A fragments 16-byte loads of the gathered rows).
-//   MODE 0: act[row] = silu(gate_e x) * (up_e x), x = h[row / top]         (bf16 out, K = width, N = ff)
+//   MODE 0: act[row] = silu(s gate_e x) * (s up_e x), x = h[row / top]     (bf16 out, K = width, N = ff;
+//           s = in_w[row], or 1 when in_w is null)
 //   MODE 1: yk[row]  = down_e act[row]                                      (fp32 out, K = ff,    N = width)
 // and `moe_combine` sums a token's rows in the order of its choices with the router weights.  No host read and no
 // data-dependent launch shape: a decode step with experts can be captured into a graph.
@@ -187,7 +196,7 @@ constexpr int GROUP_MAX_ROWS = 1024;
 template <int MODE>
 __global__ __launch_bounds__(NT) void moe_group_kernel(void* __restrict__ out, const bf16_t* __restrict__ x,
                                                        const bf16_t* __restrict__ w, const int* __restrict__ ids,
-                                                       int rows_, int K, int N, int top) {
+                                                       const float* __restrict__ in_w, int rows_, int K, int N, int top) {
   __shared__ int list[GROUP_MAX_ROWS];
   __shared__ int cnt;
   const int e = blockIdx.x;
@@ -221,8 +230,13 @@ __global__ __launch_bounds__(NT) void moe_group_kernel(void* __restrict__ out, c
         const int row = mt * 16 + 4 * grp + r;
         if (row < n) {
           const size_t at = (size_t)list[row] * N + n0 + col;
-          if constexpr (MODE == 0) reinterpret_cast<bf16_t*>(out)[at] = f2bf(ag[r] / (1.f + expf(-ag[r])) * au[r]);
-          else reinterpret_cast<float*>(out)[at] = ag[r];
+          if constexpr (MODE == 0) {
+            const float isc = in_w != nullptr ? in_w[list[row]] : 1.f;
+            const float gg = ag[r] * isc;
+            reinterpret_cast<bf16_t*>(out)[at] = f2bf(gg / (1.f + expf(-gg)) * (au[r] * isc));
+          } else {
+            reinterpret_cast<float*>(out)[at] = ag[r];
+          }
         }
       }
     }
@@ -234,7 +248,7 @@ __global__ __launch_bounds__(NT) void moe_combine_kernel(float* __restrict__ out
   const int t = blockIdx.x;
   for (int c = threadIdx.x; c < width; c += NT) {
     float s = 0.f;
-    for (int k = 0; k < top; ++k) s += wts[(size_t)t * top + k] * yk[((size_t)t * top + k) * width + c];
+    for (int k = 0; k < top; ++k) s += (wts != nullptr ? wts[(size_t)t * top + k] : 1.f) * yk[((size_t)t * top + k) * width + c];
     out[(size_t)t * width + c] = s;
   }
 }
@@ -242,40 +256,51 @@ __global__ __launch_bounds__(NT) void moe_combine_kernel(float* __restrict__ out
 }  // namespace
 
 extern "C" int ka_moe_route(int* ids, float* wts, const void* h, const float* wr, const float* correction, int T,
-                            int width, int E, int top, int groups, int keep, int f32, hipStream_t st) {
+                            int width, int E, int top, int groups, int keep, int sigmoid, int renorm, int f32,
+                            hipStream_t st) {
   if (T <= 0) return 0;
   if (E <= 0 || E > MAX_E || top <= 0 || top > MAX_TOP || top > E || groups <= 0 || E % groups || keep <= 0 || keep > groups)
     return (int)hipErrorInvalidValue;
-  if (f32) moe_route_kernel<float><<<T, NT, 0, st>>>(ids, wts, (const float*)h, wr, correction, width, E, top, groups, keep);
-  else moe_route_kernel<bf16_t><<<T, NT, 0, st>>>(ids, wts, (const bf16_t*)h, wr, correction, width, E, top, groups, keep);
+  if (f32)
+    moe_route_kernel<float><<<T, NT, 0, st>>>(ids, wts, (const float*)h, wr, correction, width, E, top, groups, keep, sigmoid,
+                                              renorm);
+  else
+    moe_route_kernel<bf16_t><<<T, NT, 0, st>>>(ids, wts, (const bf16_t*)h, wr, correction, width, E, top, groups, keep,
+                                               sigmoid, renorm);
   KA_CHECK_LAUNCH();
 }
 
 extern "C" int ka_moe_rows(float* out, void* act, const void* h, const void* w_gu, const void* w_down, const int* ids,
-                           const float* wts, int T, int width, int ff, int top, int f32, hipStream_t st) {
+                           const float* wts, int T, int width, int ff, int top, int in_scale, int f32, hipStream_t st) {
   if (T <= 0) return 0;
   if (top <= 0 || top > MAX_TOP || (size_t)width * 4 > 60 * 1024 || (size_t)top * ff * 4 > 60 * 1024)
     return (int)hipErrorInvalidValue;
   const int per = NW * FPW;
   dim3 g1(T * top, (ff + per - 1) / per), g2(T, (width + per - 1) / per);
   const size_t l1 = (size_t)width * sizeof(float), l2 = (size_t)top * ff * sizeof(float);
+  const float* w_in = in_scale ? wts : nullptr;
+  const float* w_out = in_scale ? nullptr : wts;
   if (f32) {
-    moe_gate_up_kernel<float><<<g1, NT, l1, st>>>((float*)act, (const float*)h, (const float*)w_gu, ids, width, ff, top);
-    moe_down_kernel<float><<<g2, NT, l2, st>>>(out, (const float*)act, (const float*)w_down, ids, wts, width, ff, top);
+    moe_gate_up_kernel<float><<<g1, NT, l1, st>>>((float*)act, (const float*)h, (const float*)w_gu, ids, w_in, width, ff, top);
+    moe_down_kernel<float><<<g2, NT, l2, st>>>(out, (const float*)act, (const float*)w_down, ids, w_out, width, ff, top);
   } else {
-    moe_gate_up_kernel<bf16_t><<<g1, NT, l1, st>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, ids, width, ff, top);
-    moe_down_kernel<bf16_t><<<g2, NT, l2, st>>>(out, (const bf16_t*)act, (const bf16_t*)w_down, ids, wts, width, ff, top);
+    moe_gate_up_kernel<bf16_t><<<g1, NT, l1, st>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, ids, w_in, width, ff,
+                                                   top);
+    moe_down_kernel<bf16_t><<<g2, NT, l2, st>>>(out, (const bf16_t*)act, (const bf16_t*)w_down, ids, w_out, width, ff, top);
   }
   KA_CHECK_LAUNCH();
 }
 
 // bf16 only; `act` [T * top, ff] bf16 and `yk` [T * top, width] fp32 are scratch
 extern "C" int ka_moe_grouped(float* out, void* act, float* yk, const void* h, const void* w_gu, const void* w_down,
-                              const int* ids, const float* wts, int T, int width, int ff, int top, int E, hipStream_t st) {
+                              const int* ids, const float* wts, int T, int width, int ff, int top, int E, int in_scale,
+                              hipStream_t st) {
   if (T <= 0) return 0;
   if (T * top > GROUP_MAX_ROWS || width % 32 || ff % 32 || top <= 0 || E <= 0) return (int)hipErrorInvalidValue;
-  moe_group_kernel<0><<<dim3(E, (ff + 63) / 64), NT, 0, st>>>(act, (const bf16_t*)h, (const bf16_t*)w_gu, ids, T * top, width, ff, top);
-  moe_group_kernel<1><<<dim3(E, (width + 63) / 64), NT, 0, st>>>(yk, (const bf16_t*)act, (const bf16_t*)w_down, ids, T * top, ff, width, top);
-  moe_combine_kernel<<<T, NT, 0, st>>>(out, yk, wts, width, top);
+  moe_group_kernel<0><<<dim3(E, (ff + 63) / 64), NT, 0, st>>>(act, (const bf16_t*)h, (const bf16_t*)w_gu, ids,
+                                                              in_scale ? wts : nullptr, T * top, width, ff, top);
+  moe_group_kernel<1><<<dim3(E, (width + 63) / 64), NT, 0, st>>>(yk, (const bf16_t*)act, (const bf16_t*)w_down, ids, nullptr,
+                                                                 T * top, ff, width, top);
+  moe_combine_kernel<<<T, NT, 0, st>>>(out, yk, in_scale ? nullptr : wts, width, top);
   KA_CHECK_LAUNCH();
 }

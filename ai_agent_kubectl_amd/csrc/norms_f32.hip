@@ -8,7 +8,7 @@
 //
 //   group RMS norm:  the row is cut into `groups` equal consecutive parts; part g is divided by
 //                    sqrt(mean(part_g^2) + eps); the whole row is multiplied by w.
-//   post_norm_residual:  r += ls * gnorm(y; w_post);   out_next = gnorm(r; w_next)   (optional)
+//   post_norm_residual:  r += ls * gnorm(y; w_post)  (ls null: 1);   out_next = gnorm(r; w_next)   (optional)
 //   PolyNorm:        out = a N(z) + b N(z^2) + c N(z^3) + e,  N(u) = u / sqrt(mean(u^2) + eps) per row.
 #include "common.h"
 
@@ -90,8 +90,8 @@ __global__ __launch_bounds__(NT) void group_rmsnorm_kernel(OT* __restrict__ out,
   for (int i = threadIdx.x; i < width; i += NT) stf(out + base + i, row[i] * inv[i / gsz] * w[i]);
 }
 
-template <typename AT>
-__global__ __launch_bounds__(NT) void post_norm_residual_kernel(float* __restrict__ resid, const AT* __restrict__ y,
+template <typename YT, typename AT>   // YT: the sublayer's result (fp32 for a sum of experts), AT: the next norm's output
+__global__ __launch_bounds__(NT) void post_norm_residual_kernel(float* __restrict__ resid, const YT* __restrict__ y,
                                                                 const float* __restrict__ w_post,
                                                                 const float* __restrict__ ls,
                                                                 const float* __restrict__ w_next,
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(NT) void post_norm_residual_kernel(float* __restric
   const int gsz = width / groups;
   for (int i = threadIdx.x; i < width; i += NT) {
     const float n = row[i] * inv[i / gsz] * w_post[i];
-    const float r = resid[base + i] + ls[i] * n;
+    const float r = resid[base + i] + (ls != nullptr ? ls[i] * n : n);
     resid[base + i] = r;
     row[i] = r;   // each thread rewrites only the entries it read
   }
@@ -180,16 +180,22 @@ extern "C" int ka_group_rmsnorm(void* out, const void* x, const float* w, int ro
 
 extern "C" int ka_post_norm_residual(float* resid, const void* y, const float* w_post, const float* ls,
                                      const float* w_next, void* out_next, int rows, int width, int groups, float eps,
-                                     int f32, hipStream_t st) {
+                                     int y_f32, int out_f32, hipStream_t st) {
   if (rows <= 0) return 0;
   if (!row_ok(rows, width, groups)) return (int)hipErrorInvalidValue;
   const size_t lds = row_lds(width);
-  if (f32)
-    post_norm_residual_kernel<float><<<rows, NT, lds, st>>>(resid, (const float*)y, w_post, ls, w_next, (float*)out_next,
-                                                           width, groups, eps);
+  if (y_f32 && out_f32)
+    post_norm_residual_kernel<float, float><<<rows, NT, lds, st>>>(resid, (const float*)y, w_post, ls, w_next,
+                                                                  (float*)out_next, width, groups, eps);
+  else if (y_f32)
+    post_norm_residual_kernel<float, bf16_t><<<rows, NT, lds, st>>>(resid, (const float*)y, w_post, ls, w_next,
+                                                                   (bf16_t*)out_next, width, groups, eps);
+  else if (out_f32)
+    post_norm_residual_kernel<bf16_t, float><<<rows, NT, lds, st>>>(resid, (const bf16_t*)y, w_post, ls, w_next,
+                                                                   (float*)out_next, width, groups, eps);
   else
-    post_norm_residual_kernel<bf16_t><<<rows, NT, lds, st>>>(resid, (const bf16_t*)y, w_post, ls, w_next,
-                                                            (bf16_t*)out_next, width, groups, eps);
+    post_norm_residual_kernel<bf16_t, bf16_t><<<rows, NT, lds, st>>>(resid, (const bf16_t*)y, w_post, ls, w_next,
+                                                                    (bf16_t*)out_next, width, groups, eps);
   KA_CHECK_LAUNCH();
 }
 

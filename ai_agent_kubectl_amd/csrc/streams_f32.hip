@@ -8,7 +8,9 @@
 //                   pass, and (optionally) the next sublayer's stream_norm of the new copies in the same pass.
 //
 // S = 1 with w_in = mix = out = 1 is the plain pre-norm residual.  Also here: the embedding gather into
-// the S copies with a scale, relu(z)^2, silu(gate) * up, and the per-head RMS division with an output
+// the S copies with a scale, relu(z)^2, silu(gate) * up (optionally of a row whose input was multiplied by a number
+// s: silu(s gate) * (s up)), the clamped gated unit g sigmoid(alpha g) (u + 1) with g = min(gate, limit) and
+// u = clamp(up, -limit, limit), and the per-head RMS division with an output
 // gate that closes an mLSTM (o <- o / den; out = o / rms_head(o) * w * sigmoid(g)).
 #include "rows_f32.h"
 
@@ -119,12 +121,26 @@ __global__ __launch_bounds__(NT) void relu_sq_kernel(AT* __restrict__ out, const
 }
 
 template <typename AT>
-__global__ __launch_bounds__(NT) void silu_mul_rows_kernel(AT* __restrict__ out, const AT* __restrict__ gu, int ff) {
+__global__ __launch_bounds__(NT) void silu_mul_rows_kernel(AT* __restrict__ out, const AT* __restrict__ gu,
+                                                           const float* __restrict__ row_scale, int ff) {
   const AT* g = gu + (size_t)blockIdx.x * 2 * ff;
   AT* o = out + (size_t)blockIdx.x * ff;
+  const float sc = row_scale != nullptr ? row_scale[blockIdx.x] : 1.f;
   for (int i = threadIdx.x; i < ff; i += NT) {
-    const float a = ldf(g + i);
-    stf(o + i, a / (1.f + expf(-a)) * ldf(g + ff + i));
+    const float a = ldf(g + i) * sc;
+    stf(o + i, a / (1.f + expf(-a)) * (ldf(g + ff + i) * sc));
+  }
+}
+
+template <typename AT>
+__global__ __launch_bounds__(NT) void glu_clamp_kernel(AT* __restrict__ out, const AT* __restrict__ gu, int ff, float limit,
+                                                       float alpha) {
+  const AT* g = gu + (size_t)blockIdx.x * 2 * ff;
+  AT* o = out + (size_t)blockIdx.x * ff;
+  for (int i = threadIdx.x + blockIdx.y * NT; i < ff; i += NT * gridDim.y) {
+    const float a = fminf(ldf(g + i), limit);
+    const float u = fminf(fmaxf(ldf(g + ff + i), -limit), limit);
+    stf(o + i, a / (1.f + expf(-alpha * a)) * (u + 1.f));
   }
 }
 
@@ -198,10 +214,22 @@ extern "C" int ka_relu_sq(void* out, const void* z, long n, int f32, hipStream_t
   KA_CHECK_LAUNCH();
 }
 
-extern "C" int ka_silu_mul_rows(void* out, const void* gu, int rows_, int ff, int f32, hipStream_t st) {
+// row_scale [rows] or null
+extern "C" int ka_silu_mul_rows(void* out, const void* gu, const float* row_scale, int rows_, int ff, int f32,
+                                hipStream_t st) {
   if (rows_ <= 0) return 0;
-  if (f32) silu_mul_rows_kernel<float><<<rows_, NT, 0, st>>>((float*)out, (const float*)gu, ff);
-  else silu_mul_rows_kernel<bf16_t><<<rows_, NT, 0, st>>>((bf16_t*)out, (const bf16_t*)gu, ff);
+  if (f32) silu_mul_rows_kernel<float><<<rows_, NT, 0, st>>>((float*)out, (const float*)gu, row_scale, ff);
+  else silu_mul_rows_kernel<bf16_t><<<rows_, NT, 0, st>>>((bf16_t*)out, (const bf16_t*)gu, row_scale, ff);
+  KA_CHECK_LAUNCH();
+}
+
+extern "C" int ka_glu_clamp(void* out, const void* gu, int rows_, int ff, float limit, float alpha, int f32, hipStream_t st) {
+  if (rows_ <= 0) return 0;
+  if (ff <= 0) return (int)hipErrorInvalidValue;
+  // few rows (a decode step): a row's entries are spread over several workgroups
+  const dim3 grid(rows_, rows_ < 1024 ? (ff + 4 * NT - 1) / (4 * NT) : 1);
+  if (f32) glu_clamp_kernel<float><<<grid, NT, 0, st>>>((float*)out, (const float*)gu, ff, limit, alpha);
+  else glu_clamp_kernel<bf16_t><<<grid, NT, 0, st>>>((bf16_t*)out, (const bf16_t*)gu, ff, limit, alpha);
   KA_CHECK_LAUNCH();
 }
 

@@ -16,6 +16,7 @@ from typing import Optional
 
 import torch
 
+from ..models import MIXER_FAMILIES
 from ..models.config import get_config
 from ..models.weights import ParallelInfo, build_weights
 from .engine import LLMEngine
@@ -67,7 +68,7 @@ def build_engine(opts: EngineOptions, comm=None, metrics=None) -> LLMEngine:
     dev = torch.device(opts.device)
     if dev.type == "cuda":
         # fail loudly: the GPU path never runs without the HIP kernels of the model's family
-        if getattr(cfg, "family", "llama") in ("vivepel", "kafilorn", "suvapel"):
+        if getattr(cfg, "family", "llama") in MIXER_FAMILIES:
             from ..ops._hip import require_mixers
             require_mixers()
         else:
@@ -80,7 +81,7 @@ def build_engine(opts: EngineOptions, comm=None, metrics=None) -> LLMEngine:
     family = getattr(cfg, "family", "llama")
     if dtype == torch.float32 and family in ("llama", "mixtral"):
         raise ValueError("the Llama / Mixtral kernels are bf16; float32 is served by the fp32-residual families "
-                         "(vivepel, kafilorn, suvapel)")
+                         "(%s)" % ", ".join(MIXER_FAMILIES))
     if dtype == torch.float32:   # true fp32 products: no reduced-precision matrix mode
         torch.backends.cuda.matmul.allow_tf32 = False
         torch.backends.cudnn.allow_tf32 = False

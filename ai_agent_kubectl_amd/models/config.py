@@ -664,8 +664,221 @@ def suvapel_uniform(name: str, layers: int, hidden: int, heads: int, kv_heads: i
     return SuvapelConfig(name, vocab, hidden, 1e-5, 1.0, side_dim, ls)
 
 
+# ------------------------------------------------------------------------------------------------
+# Zibinex: layers listed one by one, each x += norm(mixer(norm x)) then x += norm(ff(norm x)) with RMS norms whose
+# weights are stored around zero; a layer's mixer is latent attention with direct queries, interleaved YaRN-scaled
+# rotary positions and a sigmoid gate per head on the output, or sliding-window attention whose weights are
+# sigmoids of the score minus a logarithmic distance bias (no softmax); its feed-forward is a clamped gated unit,
+# a mixture of experts with a sigmoid router whose weight scales the expert's input, or absent.  A layer may run on
+# another layer's weights with a cache of its own.
+@dataclasses.dataclass(frozen=True)
+class GatedLatentAttentionSpec:
+    """Softmax attention over a cached latent [kv_rank] plus one rotated key part [rot_dim] shared by the heads;
+    queries are projected directly, head by head [dim unrotated | rot_dim rotated]; rotary pairs are (2i, 2i + 1);
+    head h's result is multiplied by sigmoid of one gate logit per token and head."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    window: int                 # position i sees j with 0 <= i - j < window (0: all of 0 .. i)
+    rot: RotarySpec
+    scale: float
+    kind: str = "latent_attention"
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "GatedLatentAttentionSpec":
+        mask = m.get("mask") or {}
+        spec = cls(heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]),
+                   kv_rank=int(m["kv_rank"]), window=int(mask.get("size") or 0), rot=RotarySpec.from_dict(m.get("rot")),
+                   scale=float(m["scale"]))
+        if spec.rot.dims % 2 or spec.rot.dims > spec.rot_dim or spec.window < 0 or min(spec.heads, spec.kv_rank, spec.vdim) < 1:
+            raise ValueError(f"bad latent attention sizes: {spec}")
+        return spec
+
+    def to_dict(self) -> dict:
+        d = {"heads": self.heads, "dim": self.dim, "rot_dim": self.rot_dim, "vdim": self.vdim, "kv_rank": self.kv_rank,
+             "scale": self.scale}
+        if self.window:
+            d["mask"] = {"size": self.window}
+        if self.rot.dims:
+            d["rot"] = self.rot.to_dict()
+        return d
+
+    def cache_entries(self) -> int:
+        return self.kv_rank + self.rot_dim
+
+
+@dataclasses.dataclass(frozen=True)
+class SigmoidAttentionSpec:
+    """Attention with grouped keys / values, biases on q, k, v, a per-head RMS norm of q and k, no rotation, a
+    sliding window, and weights sigmoid(score - r1 ln(1 + r2 distance) + pb) that are not normalised over the keys
+    (r1, r2, pb: one learned number per head each)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    window: int                 # position i sees j with 0 <= i - j < window (0: all of 0 .. i)
+    scale: float
+    kind: str = "attention"
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "SigmoidAttentionSpec":
+        mask = m.get("mask") or {}
+        spec = cls(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                   window=int(mask.get("size") or 0), scale=float(m["scale"]))
+        if spec.kv_heads < 1 or spec.heads % spec.kv_heads or spec.window < 0 or min(spec.dim, spec.vdim) < 1:
+            raise ValueError(f"bad attention sizes: {spec}")
+        return spec
+
+    def to_dict(self) -> dict:
+        d = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale}
+        if self.window:
+            d["mask"] = {"size": self.window}
+        return d
+
+    def cache_entries(self) -> int:
+        return self.kv_heads * (self.dim + self.vdim)
+
+
+@dataclasses.dataclass(frozen=True)
+class ClampedFeedForwardSpec:
+    """dense: down(g sigmoid(1.702 g) (u + 1)) with g = min(gate h, limit), u = clamp(up h, -limit, limit).
+    moe: `experts` gated experts of width ff (silu), the `top` largest sigmoid router scores chosen per token; a
+    chosen expert's score multiplies its input, and the results are summed as they are."""
+    kind: str                   # "dense" | "moe"
+    ff: int
+    limit: float = 0.0
+    experts: int = 0
+    top: int = 0
+
+    GLU_ALPHA = 1.702           # the sigmoid's slope in the dense unit
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "ClampedFeedForwardSpec":
+        if m["kind"] == "dense":
+            return cls("dense", int(m["ff"]), limit=float(m["limit"]))
+        if m["kind"] != "moe":
+            raise ValueError(f"unknown feed-forward kind {m['kind']!r}")
+        spec = cls("moe", int(m["expert"]["ff"]), experts=int(m["router"]["experts"]), top=int(m["router"]["top"]))
+        if not 0 < spec.top <= spec.experts:
+            raise ValueError(f"bad router: {spec}")
+        return spec
+
+    def to_dict(self) -> dict:
+        if self.kind == "dense":
+            return {"kind": "dense", "ff": self.ff, "limit": self.limit}
+        return {"kind": "moe", "expert": {"ff": self.ff}, "router": {"experts": self.experts, "top": self.top}}
+
+
+@dataclasses.dataclass(frozen=True)
+class ZibinexLayer:
+    mixer: object               # GatedLatentAttentionSpec | SigmoidAttentionSpec
+    mlp: Optional[ClampedFeedForwardSpec]
+    weights_of: int = -1        # >= 0: no tensors of its own, runs on that layer's; its cache is its own
+
+
+_ZIBINEX_MIXERS = {"latent_attention": GatedLatentAttentionSpec, "attention": SigmoidAttentionSpec}
+
+
+@dataclasses.dataclass(frozen=True)
+class ZibinexConfig:
+    name: str
+    vocab_size: int
+    hidden: int
+    norm_eps: float
+    layers: Tuple[ZibinexLayer, ...]
+    max_position: int = 1 << 20
+    tokenizer: str = "llama3"
+    family: str = "zibinex"
+    tie_embeddings: bool = True
+    is_moe: bool = False        # its experts are not sharded: the engine's expert-parallel wiring does not apply
+    has_state: bool = False
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def owner(self, i: int) -> int:
+        """The layer whose tensors layer i runs on."""
+        return self.layers[i].weights_of if self.layers[i].weights_of >= 0 else i
+
+    @classmethod
+    def from_dict(cls, d: dict, name: str = "zibinex") -> "ZibinexConfig":
+        layers = []
+        for i, L in enumerate(d["layers"]):
+            if L["type"] not in _ZIBINEX_MIXERS:
+                raise ValueError(f"layer {i}: unknown mixer type {L['type']!r}")
+            wo = L.get("weights_of")
+            layers.append(ZibinexLayer(_ZIBINEX_MIXERS[L["type"]].from_dict(L["mixer"]),
+                                       ClampedFeedForwardSpec.from_dict(L["mlp"]) if L.get("mlp") is not None else None,
+                                       -1 if wo is None else int(wo)))
+        for i, L in enumerate(layers):
+            if L.weights_of >= 0:
+                src = layers[L.weights_of] if L.weights_of < len(layers) and L.weights_of != i else None
+                if src is None or src.weights_of >= 0 or (src.mixer, src.mlp) != (L.mixer, L.mlp):
+                    raise ValueError(f"layer {i}: weights_of {L.weights_of} must name another layer of the same sizes "
+                                     "that has tensors of its own")
+        return cls(name=name, vocab_size=int(d["vocab"]), hidden=int(d["width"]), norm_eps=float(d["norm"]["eps"]),
+                   layers=tuple(layers))
+
+    def to_dict(self) -> dict:
+        out = []
+        for L in self.layers:
+            e = {"type": L.mixer.kind, "mixer": L.mixer.to_dict(), "mlp": L.mlp.to_dict() if L.mlp else None}
+            if L.weights_of >= 0:
+                e["weights_of"] = L.weights_of
+            out.append(e)
+        return {"architecture": "Zibinex", "vocab": self.vocab_size, "width": self.hidden, "norm": {"eps": self.norm_eps},
+                "layers": out}
+
+    def num_params(self) -> int:
+        h = self.hidden
+        n = self.vocab_size * h + h
+        for L in self.layers:
+            if L.weights_of >= 0:
+                continue
+            m, f = L.mixer, L.mlp
+            if m.kind == "latent_attention":
+                n += h * (m.heads * (m.dim + m.rot_dim + 1) + m.kv_rank + m.rot_dim) + m.kv_rank
+                n += m.heads * (m.kv_rank * (m.dim + m.vdim) + m.vdim * h)
+            else:
+                n += (h + 1) * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + 2 * m.dim + 3 * m.heads + m.heads * m.vdim * h
+            n += 2 * h
+            if f is not None:
+                n += 2 * h + (3 * h * f.ff if f.kind == "dense" else f.experts * (3 * h * f.ff + h))
+        return n
+
+    def default_step_tokens(self) -> int:
+        return 8192
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        """Paged cache per token: every layer's own entries, also of a layer that runs on another's weights."""
+        return max(1, sum(L.mixer.cache_entries() * dtype_bytes for L in self.layers))
+
+
+def zibinex_uniform(name: str, layers: int, hidden: int, heads: int, kv_heads: int, dim: int, ff: int, vocab: int,
+                    window: int = 1024, kv_rank: int = 0, rot_dim: int = 0, experts: int = 8, top: int = 2,
+                    expert_ff: int = 0, share: bool = False, limit: float = 7.0) -> ZibinexConfig:
+    """A regular Zibinex (benchmarks, tests): latent attention and sliding sigmoid attention in turn; the first layer
+    has the dense feed-forward, the others experts; share: every latent layer after the second layer's runs on its
+    weights."""
+    rot_dim = rot_dim or dim // 2
+    rot = RotarySpec(rot_dim, 10000.0, 8.0, 4096, 32.0, 1.0)
+    lat = GatedLatentAttentionSpec(heads, dim, rot_dim, dim, kv_rank or hidden // 4, 0, rot, (dim + rot_dim) ** -0.5)
+    att = SigmoidAttentionSpec(heads, kv_heads, dim, dim, window, dim ** -0.5)
+    dense = ClampedFeedForwardSpec("dense", ff, limit=limit)
+    moe = ClampedFeedForwardSpec("moe", expert_ff or ff // 4, experts=experts, top=top)
+    out = []
+    for i in range(layers):
+        wo = 2 if share and i % 2 == 0 and i > 2 else -1
+        out.append(ZibinexLayer(lat if i % 2 == 0 else att, dense if i == 0 else moe, wo))
+    return ZibinexConfig(name, vocab, hidden, 1e-6, tuple(out))
+
+
 # config.json "architecture" -> parser of the file's dict
-ARCHITECTURES = {"Vivepel": VivepelConfig.from_dict, "Kafilorn": KafilornConfig.from_dict, "Suvapel": SuvapelConfig.from_dict}
+ARCHITECTURES = {"Vivepel": VivepelConfig.from_dict, "Kafilorn": KafilornConfig.from_dict, "Suvapel": SuvapelConfig.from_dict,
+                 "Zibinex": ZibinexConfig.from_dict}
 
 
 def load_config_dir(path: str):
@@ -712,6 +925,11 @@ PRESETS: Dict[str, ModelConfig] = {
     "tiny-suvapel": suvapel_uniform("tiny-suvapel", 3, 128, 4, 2, 32, 192, 384, window=24, keep_first=3, side_dim=16,
                                     conv=3, every=3, low_rank=8),
     "suvapel-4k-2l": suvapel_uniform("suvapel-4k-2l", 2, 4096, 32, 8, 128, 14336, 128256),
+    # Zibinex at a small size (CPU tests) and at a Llama-3-8B-like width (bench.py --arch-compare)
+    "tiny-zibinex": zibinex_uniform("tiny-zibinex", 5, 128, 4, 2, 24, 256, 384, window=20, kv_rank=40, rot_dim=8,
+                                    experts=6, top=2, expert_ff=64, share=True, limit=1.25),
+    "zibinex-4k-2l": zibinex_uniform("zibinex-4k-2l", 2, 4096, 32, 8, 128, 14336, 128256, kv_rank=512, rot_dim=64,
+                                     expert_ff=3584),
 }
 
 

@@ -688,6 +688,154 @@ def load_suvapel_safetensors(path: str, cfg, device="cpu", dtype=torch.bfloat16)
     return W
 
 
+# ------------------------------------------------------------------------------------------------
+# Zibinex.  Engine layout per layer that has tensors of its own, `layers.<i>.` (activation dtype unless marked fp32;
+# a layer with weights_of has no entries, the model points it at its owner's):
+#   norm1, norm1b, norm2, norm2b [W] fp32, stored as 1 + w (the checkpoint keeps the weights around zero)
+#   latent attention:  w_in [dkv rows (kv_rank + rot_dim); q rows (H * (dim + rot_dim)); g rows (H); zero rows up to a
+#           multiple of 8, W] (one GEMM; `zibinex_columns`), kv_norm [kv_rank] fp32, w_uk [H, dim, kv_rank],
+#           w_uv [H, vdim, kv_rank], inv_freq [rot dims / 2] fp32 (YaRN-scaled, float64 rounded once), wo [W, H * vdim]
+#   attention:  w_qkv [q; k; v rows, W] + b_qkv (one GEMM), q_norm / k_norm [dim] fp32, dist [3, H] fp32 (the rows
+#           r1, r2, pb), wo [W, H * vdim]
+#   dense feed-forward:  w_gu [gate rows; up rows, W], w_down [W, ff]
+#   experts:  w_router [E, W] fp32, w_gu_e [E, 2 ff, W] (gate rows, then up rows), w_dn_e [E, W, ff]
+# The LM head is the embedding table.
+_ZIBINEX_F32 = ("norm1", "norm1b", "norm2", "norm2b", "kv_norm", "inv_freq", "q_norm", "k_norm", "dist", "w_router")
+
+
+def zibinex_columns(m) -> Dict[str, int]:
+    """Column offsets of a latent-attention layer's fused input projection."""
+    q = m.kv_rank + m.rot_dim
+    g = q + m.heads * (m.dim + m.rot_dim)
+    return {"kv": 0, "q": q, "g": g, "total": _pad8(g + m.heads)}
+
+
+def _zibinex_pack(cfg, get, device, dtype) -> Dict[str, torch.Tensor]:
+    def one_plus(name):
+        return 1.0 + get(name).float()
+
+    W: Dict[str, torch.Tensor] = {"embed": get("embed"), "norm": one_plus("final.norm")}
+    for i, L in enumerate(cfg.layers):
+        if L.weights_of >= 0:
+            continue
+        p, c, m, f = f"layers.{i}.", f"l{i}.", L.mixer, L.mlp
+        for k in ("norm1", "norm1b") + (("norm2", "norm2b") if f is not None else ()):
+            W[p + k] = one_plus(c + k)
+        if m.kind == "latent_attention":
+            rows = torch.cat([get(c + "mix.dkv"), get(c + "mix.q"), get(c + "mix.g")])
+            pad = zibinex_columns(m)["total"] - rows.shape[0]
+            W[p + "w_in"] = torch.cat([rows, rows.new_zeros((pad, rows.shape[1]))]) if pad else rows
+            W[p + "kv_norm"] = get(c + "mix.dkv.norm")
+            W[p + "w_uk"] = get(c + "mix.uk").view(m.heads, m.dim, m.kv_rank)
+            W[p + "w_uv"] = get(c + "mix.uv").view(m.heads, m.vdim, m.kv_rank)
+            W[p + "inv_freq"] = torch.tensor(m.rot.frequencies()[0], dtype=torch.float64)
+        else:
+            W[p + "w_qkv"] = torch.cat([get(c + "mix.q"), get(c + "mix.k"), get(c + "mix.v")])
+            W[p + "b_qkv"] = torch.cat([get(c + "mix.q.b"), get(c + "mix.k.b"), get(c + "mix.v.b")])
+            W[p + "q_norm"], W[p + "k_norm"] = get(c + "mix.q.norm"), get(c + "mix.k.norm")
+            W[p + "dist"] = torch.stack([get(c + "mix.r1"), get(c + "mix.r2"), get(c + "mix.pb")])
+        W[p + "wo"] = get(c + "mix.o")
+        if f is None:
+            continue
+        if f.kind == "dense":
+            W[p + "w_gu"], W[p + "w_down"] = torch.cat([get(c + "mlp.gate"), get(c + "mlp.up")]), get(c + "mlp.down")
+        else:
+            W[p + "w_router"] = get(c + "mlp.router")
+            W[p + "w_gu_e"] = torch.stack([torch.cat([get(c + f"mlp.e{e}.gate"), get(c + f"mlp.e{e}.up")])
+                                           for e in range(f.experts)])
+            W[p + "w_dn_e"] = torch.stack([get(c + f"mlp.e{e}.down") for e in range(f.experts)])
+    out = {}
+    for k, v in W.items():
+        f32 = k == "norm" or k.rsplit(".", 1)[-1] in _ZIBINEX_F32
+        out[k] = v.to(device=device, dtype=torch.float32 if f32 else dtype).contiguous()
+    out["lm_head"] = out["embed"]
+    return out
+
+
+def zibinex_check_shapes(cfg, W: Dict[str, torch.Tensor]) -> None:
+    """Every tensor of the engine layout has the shape the configuration implies."""
+    h, V = cfg.hidden, cfg.vocab_size
+    want = {"embed": (V, h), "norm": (h,)}
+    for i, L in enumerate(cfg.layers):
+        if L.weights_of >= 0:
+            continue
+        p, m, f = f"layers.{i}.", L.mixer, L.mlp
+        want.update({p + "norm1": (h,), p + "norm1b": (h,), p + "wo": (h, m.heads * m.vdim)})
+        if m.kind == "latent_attention":
+            want.update({p + "w_in": (zibinex_columns(m)["total"], h), p + "kv_norm": (m.kv_rank,),
+                         p + "w_uk": (m.heads, m.dim, m.kv_rank), p + "w_uv": (m.heads, m.vdim, m.kv_rank),
+                         p + "inv_freq": (m.rot.dims // 2,)})
+        else:
+            n = m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)
+            want.update({p + "w_qkv": (n, h), p + "b_qkv": (n,), p + "q_norm": (m.dim,), p + "k_norm": (m.dim,),
+                         p + "dist": (3, m.heads)})
+        if f is not None:
+            want.update({p + "norm2": (h,), p + "norm2b": (h,)})
+            if f.kind == "dense":
+                want.update({p + "w_gu": (2 * f.ff, h), p + "w_down": (h, f.ff)})
+            else:
+                want.update({p + "w_router": (f.experts, h), p + "w_gu_e": (f.experts, 2 * f.ff, h),
+                             p + "w_dn_e": (f.experts, h, f.ff)})
+    for k, shp in want.items():
+        if k not in W or tuple(W[k].shape) != shp:
+            raise ValueError(f"tensor {k}: expected shape {shp}, found {tuple(W[k].shape) if k in W else None}")
+
+
+def zibinex_checkpoint_tensors(cfg, seed: int = 0, dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Random tensors under the checkpoint's own names (what a Zibinex model.safetensors holds)."""
+    g = torch.Generator().manual_seed(_seed(seed, "zibinex") & 0x7FFFFFFF)
+    h, V = cfg.hidden, cfg.vocab_size
+
+    def mat(o, i, std=None):
+        return (torch.randn(o, i, generator=g) * (std if std is not None else i ** -0.5)).to(dtype)
+
+    def vec(n, lo=0.75, hi=1.25):
+        return (lo + (hi - lo) * torch.rand(n, generator=g)).to(dtype)
+
+    T = {"embed": mat(V, h, 1.0), "final.norm": vec(h, -0.25, 0.25)}
+    for i, L in enumerate(cfg.layers):
+        if L.weights_of >= 0:
+            continue
+        c, m, f = f"l{i}.", L.mixer, L.mlp
+        for k in ("norm1", "norm1b") + (("norm2", "norm2b") if f is not None else ()):
+            T[c + k] = vec(h, -0.25, 0.25)
+        if m.kind == "latent_attention":
+            T[c + "mix.q"] = mat(m.heads * (m.dim + m.rot_dim), h)
+            T[c + "mix.dkv"], T[c + "mix.dkv.norm"] = mat(m.kv_rank + m.rot_dim, h), vec(m.kv_rank)
+            T[c + "mix.uk"], T[c + "mix.uv"] = mat(m.heads * m.dim, m.kv_rank), mat(m.heads * m.vdim, m.kv_rank)
+            T[c + "mix.g"] = mat(m.heads, h)
+        else:
+            for k, n in (("q", m.heads * m.dim), ("k", m.kv_heads * m.dim), ("v", m.kv_heads * m.vdim)):
+                T[c + "mix." + k], T[c + f"mix.{k}.b"] = mat(n, h), (torch.randn(n, generator=g) * 0.1).to(dtype)
+            T[c + "mix.q.norm"], T[c + "mix.k.norm"] = vec(m.dim), vec(m.dim)
+            T[c + "mix.r1"], T[c + "mix.r2"] = vec(m.heads, 0.25, 1.0), vec(m.heads, 0.1, 1.0)
+            T[c + "mix.pb"] = vec(m.heads, -3.0, -1.0)
+        T[c + "mix.o"] = mat(h, m.heads * m.vdim)
+        if f is not None and f.kind == "dense":
+            T[c + "mlp.gate"], T[c + "mlp.up"], T[c + "mlp.down"] = mat(f.ff, h), mat(f.ff, h), mat(h, f.ff)
+        elif f is not None:
+            T[c + "mlp.router"] = mat(f.experts, h, 2.0 * h ** -0.5)
+            for e in range(f.experts):
+                n = f"mlp.e{e}."
+                T[c + n + "gate"], T[c + n + "up"], T[c + n + "down"] = mat(f.ff, h), mat(f.ff, h), mat(h, f.ff)
+    return T
+
+
+def zibinex_random_weights(cfg, seed: int = 0, device="cpu", dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Random-init Zibinex weights: drawn in bf16 (as a checkpoint stores them), packed for `dtype`."""
+    T = zibinex_checkpoint_tensors(cfg, seed)
+    W = _zibinex_pack(cfg, T.__getitem__, device, dtype)
+    zibinex_check_shapes(cfg, W)
+    return W
+
+
+def load_zibinex_safetensors(path: str, cfg, device="cpu", dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """A Zibinex checkpoint (a file, or a folder holding model.safetensors / *.safetensors)."""
+    W = _zibinex_pack(cfg, _safetensors_getter(path), device, dtype)
+    zibinex_check_shapes(cfg, W)
+    return W
+
+
 def build_weights(spec: str, cfg: ModelConfig, par: ParallelInfo, device="cpu", dtype=torch.bfloat16):
     if getattr(cfg, "family", "") == "vivepel":
         if par.tp_size != 1 or par.ep_size != 1:
@@ -710,6 +858,13 @@ def build_weights(spec: str, cfg: ModelConfig, par: ParallelInfo, device="cpu", 
             seed = int(spec.split(":", 1)[1]) if ":" in spec else 0
             return suvapel_random_weights(cfg, seed=seed, device=device, dtype=dtype)
         return load_suvapel_safetensors(spec, cfg, device=device, dtype=dtype)
+    if getattr(cfg, "family", "") == "zibinex":
+        if par.tp_size != 1 or par.ep_size != 1:
+            raise ValueError("Zibinex runs at TP = 1 (data parallel replicas scale it out)")
+        if spec.startswith("random"):
+            seed = int(spec.split(":", 1)[1]) if ":" in spec else 0
+            return zibinex_random_weights(cfg, seed=seed, device=device, dtype=dtype)
+        return load_zibinex_safetensors(spec, cfg, device=device, dtype=dtype)
     if spec.startswith("random"):
         seed = int(spec.split(":", 1)[1]) if ":" in spec else 0
         return random_weights(cfg, par, seed=seed, device=device, dtype=dtype)

@@ -109,7 +109,7 @@ _SIGS = {
 _MIX_SIGS = {
     "ka_embed_f32": [P, P, P, I, I, I, I, P],
     "ka_group_rmsnorm": [P, P, P, I, I, I, F, I, I, P],
-    "ka_post_norm_residual": [P, P, P, P, P, P, I, I, I, F, I, P],
+    "ka_post_norm_residual": [P, P, P, P, P, P, I, I, I, F, I, I, P],
     "ka_polynorm": [P, P, P, I, I, F, I, P],
     "ka_headnorm_rope_append": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, P],
     "ka_chunk_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, F, I, P],
@@ -119,25 +119,27 @@ _MIX_SIGS = {
     "ka_stream_norm": [P, P, P, P, I, I, I, F, I, P],
     "ka_stream_update": [P, P, P, P, P, P, P, I, I, I, F, I, I, P],
     "ka_relu_sq": [P, P, ctypes.c_long, I, P],
-    "ka_silu_mul_rows": [P, P, I, I, I, P],
+    "ka_silu_mul_rows": [P, P, P, I, I, I, P],
+    "ka_glu_clamp": [P, P, I, I, F, F, I, P],
     "ka_headnorm_gate": [P, P, P, P, I, I, P, I, I, I, F, I, I, P],
     "ka_mlstm_gates": [P, P, P, P, I, I, I, F, I, P],
     "ka_mlstm_gates_mfma": [P, P, P, P, I, I, I, F, P],
     "ka_mlstm_scan": [P, P, P, I, I, I, I, P, P, P, P, P, P, P, I, P, I, I, I, F, I, P],
-    "ka_latent_prep": [P, P, I, I, I, I, I, P, P, P, P, P, P, I, F, I, P],
-    "ka_rope_split_q": [P, P, P, P, P, I, I, I, I, I, I, P],
+    "ka_latent_prep": [P, P, I, I, I, I, I, P, P, P, P, P, P, I, F, I, F, I, P],
+    "ka_rope_split_q": [P, P, P, I, I, P, P, I, I, I, I, I, I, F, I, P],
+    "ka_head_gate": [P, P, P, I, I, I, I, I, I, P],
     "ka_window_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
-    "ka_moe_route": [P, P, P, P, P, I, I, I, I, I, I, I, P],
-    "ka_moe_rows": [P, P, P, P, P, P, P, I, I, I, I, I, P],
-    "ka_moe_grouped": [P, P, P, P, P, P, P, P, I, I, I, I, I, P],
+    "ka_moe_route": [P, P, P, P, P, I, I, I, I, I, I, I, I, I, P],
+    "ka_moe_rows": [P, P, P, P, P, P, P, I, I, I, I, I, I, P],
+    "ka_moe_grouped": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
     "ka_dyt_norm": [P, P, P, P, P, I, I, I, P],
     "ka_residual_mix": [P, P, P, P, F, F, F, P, P, P, P, P, I, I, I, I, P],
     "ka_rms_residual": [P, P, P, F, F, P, P, P, P, I, I, I, I, P],
     "ka_gelu_gate_embed": [P, P, P, P, I, I, I, I, I, I, P],
     "ka_silu_mul_bias": [P, P, I, I, I, P, I, I, P],
     "ka_short_conv": [P, P, I, I, I, P, I, P, P, P, I, P, I, I, I, P],
-    "ka_rope_append": [P, P, P, F, P, P, P, P, I, I, I, I, I, I, I, I, P],
-    "ka_sliding_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, I, I, F, I, I, P],
+    "ka_rope_append": [P, P, P, F, P, P, P, P, I, I, I, I, I, I, I, P, P, F, I, P],
+    "ka_sliding_attention": [P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, I, I, F, P, I, I, P],
     "ka_sliding_attention_tile_ok": [I, I, I, I, I],
     "ka_delta_prep": [P, P, P, P, I, P, I, I, P, I, I, P, P, I, I, I, I, I, I, P],
     "ka_delta_scan": [P, P, P, I, I, P, P, P, P, P, I, P, I, I, I, I, I, I, I, P],

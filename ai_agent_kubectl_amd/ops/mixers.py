@@ -5,7 +5,10 @@ streams (hyper-connections) with LayerNorm, the mLSTM gates and recurrence over 
 with a sliding window and a learned sink, squared ReLU, and expert routing in groups with a choice correction.
 `models/suvapel.py`: Dynamic-Tanh norm and scaled residual sums, a gated token input, short convolutions over state
 slots, rotary positions from a frequency table, sliding-window attention that keeps the first tokens with a per-head
-gate, and the gated delta rule with a decay per head or per key channel.
+gate, and the gated delta rule with a decay per head or per key channel.  `models/zibinex.py`: latent attention with
+directly projected queries, interleaved rotary pairs and a per-head output gate, per-head norms before the cache
+append, attention weights that are sigmoids of the score minus a logarithmic distance bias, a clamped gated unit, and
+a sigmoid router whose weights scale the experts' inputs; each an option of the op it resembles.
 
 Dispatch follows `ops/__init__.py`: a GPU tensor goes to the HIP kernel (the `csrc/*.hip` sources tagged
 `KA_HIP_LIB: mixers`, built into `ops/lib/libkagent_mixers.so`) and raises if that library is
@@ -74,19 +77,22 @@ def group_rmsnorm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float, out
     return out
 
 
-def post_norm_residual(resid: torch.Tensor, y: torch.Tensor, w_post: torch.Tensor, ls: torch.Tensor,
-                       w_next: Optional[torch.Tensor], groups: int, eps: float) -> Optional[torch.Tensor]:
-    """resid += ls * gnorm(y; w_post), in place; returns gnorm(resid; w_next) in y's dtype (None without w_next)."""
+def post_norm_residual(resid: torch.Tensor, y: torch.Tensor, w_post: torch.Tensor, ls: Optional[torch.Tensor],
+                       w_next: Optional[torch.Tensor], groups: int, eps: float, out_dtype=None) -> Optional[torch.Tensor]:
+    """resid += ls * gnorm(y; w_post), in place (ls None: no layer scale); returns gnorm(resid; w_next) in out_dtype
+    (default: y's dtype; y may be an fp32 sum in a bf16 engine), None without w_next."""
+    out_dtype = out_dtype or y.dtype
     if _ref(y):
-        return ref.post_norm_residual(resid, y, w_post, ls, w_next, groups, eps)
+        return ref.post_norm_residual(resid, y, w_post, ls, w_next, groups, eps, out_dtype)
     lib = require_mixers()
     rows, width = y.shape
     assert resid.dtype == torch.float32 and resid.shape == y.shape and resid.is_contiguous() and y.is_contiguous()
-    assert w_post.dtype == torch.float32 and ls.dtype == torch.float32 and width % groups == 0
-    assert w_post.shape[0] == width and ls.shape[0] == width and (w_next is None or w_next.shape[0] == width)
-    out = torch.empty_like(y) if w_next is not None else None
+    assert w_post.dtype == torch.float32 and (ls is None or ls.dtype == torch.float32) and width % groups == 0
+    assert w_post.shape[0] == width and (ls is None or ls.shape[0] == width) and (w_next is None or w_next.shape[0] == width)
+    out = torch.empty((rows, width), dtype=out_dtype, device=y.device) if w_next is not None else None
     check(lib.ka_post_norm_residual(_p(resid), _p(y), _p(w_post), _p(ls), _p(w_next), _p(out), rows, width, groups,
-                                    float(eps), _f32(y), _stream()), "post_norm_residual")
+                                    float(eps), _f32(y), 1 if out_dtype == torch.float32 else 0, _stream()),
+          "post_norm_residual")
     return out
 
 
@@ -232,15 +238,30 @@ def relu_sq(z: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def silu_mul(gu: torch.Tensor) -> torch.Tensor:
-    """[T, 2 ff] = gate | up -> silu(gate) * up [T, ff] (bf16 or fp32)."""
+def silu_mul(gu: torch.Tensor, row_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """[T, 2 ff] = gate | up -> silu(gate) * up [T, ff] (bf16 or fp32).  row_scale [T] fp32: the rows' inputs were
+    to be multiplied by these numbers before the two projections; as those are linear, silu(s gate) * (s up)."""
     if _ref(gu):
-        return ref.silu_mul(gu)
+        return ref.silu_mul(gu) if row_scale is None else ref.silu_mul_scaled(gu, row_scale)
+    lib = require_mixers()
+    T, two = gu.shape
+    assert gu.is_contiguous() and two % 2 == 0
+    assert row_scale is None or (row_scale.dtype == torch.float32 and row_scale.shape == (T,) and row_scale.is_contiguous())
+    out = torch.empty((T, two // 2), dtype=gu.dtype, device=gu.device)
+    check(lib.ka_silu_mul_rows(_p(out), _p(gu), _p(row_scale), T, two // 2, _f32(gu), _stream()), "silu_mul_rows")
+    return out
+
+
+def glu_clamp(gu: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    """[T, 2 ff] = gate | up -> g sigmoid(alpha g) (u + 1) [T, ff] with g = min(gate, limit) and
+    u = clamp(up, -limit, limit)."""
+    if _ref(gu):
+        return ref.glu_clamp(gu, limit, alpha)
     lib = require_mixers()
     T, two = gu.shape
     assert gu.is_contiguous() and two % 2 == 0
     out = torch.empty((T, two // 2), dtype=gu.dtype, device=gu.device)
-    check(lib.ka_silu_mul_rows(_p(out), _p(gu), T, two // 2, _f32(gu), _stream()), "silu_mul_rows")
+    check(lib.ka_glu_clamp(_p(out), _p(gu), T, two // 2, float(limit), float(alpha), _f32(gu), _stream()), "glu_clamp")
     return out
 
 
@@ -315,41 +336,63 @@ def headnorm_gate(o: torch.Tensor, proj: torch.Tensor, g_off: int, w: torch.Tens
     return out
 
 
-def latent_prep(proj: torch.Tensor, Q: int, R: int, Dr: int, w_q: torch.Tensor, w_kv: Optional[torch.Tensor],
+def latent_prep(proj: torch.Tensor, Q: int, R: int, Dr: int, w_q: Optional[torch.Tensor], w_kv: Optional[torch.Tensor],
                 inv_freq: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, cache: Optional[torch.Tensor],
-                rot_dims: int, eps: float) -> torch.Tensor:
-    """Rows [query latent Q | key/value latent R | rotated key part Dr] -> the RMS-normed query latent [T, Q];
-    with a cache [NB, BS, R + Dr], the normed latent and the rotated key part are appended at `slots`."""
+                rot_dims: int, eps: float, interleaved: bool = False, mag: float = 1.0) -> Optional[torch.Tensor]:
+    """Rows [query latent Q | key/value latent R | rotated key part Dr] -> the RMS-normed query latent [T, Q] (Q = 0,
+    a model that projects its queries directly: None); with a cache [NB, BS, R + Dr], the normed latent and the
+    rotated key part are appended at `slots`.  Rotary pairs are (i, i + rot_dims / 2), or (2i, 2i + 1) when
+    interleaved; cos and sin are multiplied by `mag`."""
     if _ref(proj):
-        return ref.latent_prep(proj, Q, R, Dr, w_q, w_kv, inv_freq, positions, slots, cache, rot_dims, eps)
+        return ref.latent_prep(proj, Q, R, Dr, w_q, w_kv, inv_freq, positions, slots, cache, rot_dims, eps, interleaved, mag)
     lib = require_mixers()
     T, P = proj.shape
-    assert proj.is_contiguous() and w_q.dtype == torch.float32 and w_q.numel() == Q
+    assert proj.is_contiguous() and (Q == 0 or (w_q.dtype == torch.float32 and w_q.numel() == Q))
     assert positions.dtype == torch.int32 and slots.dtype == torch.int32 and positions.shape[0] >= T and slots.shape[0] >= T
     if cache is not None:
         assert cache.dtype == proj.dtype and cache.shape[2] == R + Dr and cache.is_contiguous() and P >= Q + R + Dr
         assert w_kv.dtype == torch.float32 and w_kv.numel() == R and inv_freq.dtype == torch.float32
         assert inv_freq.numel() * 2 == rot_dims
-    cq = torch.empty((T, Q), dtype=proj.dtype, device=proj.device)
+    cq = torch.empty((T, Q), dtype=proj.dtype, device=proj.device) if Q else None
     check(lib.ka_latent_prep(_p(cq), _p(proj), T, P, Q, R, Dr, _p(w_q), _p(w_kv), _p(inv_freq), _p(positions), _p(slots),
-                             _p(cache), rot_dims, float(eps), _f32(proj), _stream()), "latent_prep")
+                             _p(cache), rot_dims, float(eps), int(bool(interleaved)), float(mag), _f32(proj), _stream()),
+          "latent_prep")
     return cq
 
 
 def rope_split_q(q: torch.Tensor, inv_freq: torch.Tensor, positions: torch.Tensor, H: int, D: int, Dr: int,
-                 rot_dims: int):
-    """q [T, H * (D + Dr)] -> (unrotated parts [H, T, D] in q's dtype, rotated parts after rotary [T, H, Dr] fp32)."""
+                 rot_dims: int, interleaved: bool = False, mag: float = 1.0, off: int = 0):
+    """The columns off .. off + H * (D + Dr) of q's rows (q may be a fused projection) -> (unrotated parts [H, T, D]
+    in q's dtype, rotated parts after rotary [T, H, Dr] fp32).  Rotary as in `latent_prep`."""
     if _ref(q):
-        return ref.rope_split_q(q, inv_freq, positions, H, D, Dr, rot_dims)
+        return ref.rope_split_q(q, inv_freq, positions, H, D, Dr, rot_dims, interleaved, mag, off)
     lib = require_mixers()
-    T = q.shape[0]
-    assert q.is_contiguous() and q.shape[1] == H * (D + Dr) and positions.dtype == torch.int32 and positions.shape[0] >= T
-    assert inv_freq.dtype == torch.float32 and inv_freq.numel() * 2 == rot_dims
+    T, P = q.shape
+    assert q.is_contiguous() and 0 <= off and off + H * (D + Dr) <= P and positions.dtype == torch.int32
+    assert positions.shape[0] >= T and (rot_dims == 0 or (inv_freq.dtype == torch.float32 and inv_freq.numel() * 2 == rot_dims))
     qn = torch.empty((H, T, D), dtype=q.dtype, device=q.device)
     qr = torch.empty((T, H, Dr), dtype=torch.float32, device=q.device)
-    check(lib.ka_rope_split_q(_p(qn), _p(qr), _p(q), _p(inv_freq), _p(positions), T, H, D, Dr, rot_dims, _f32(q), _stream()),
-          "rope_split_q")
+    check(lib.ka_rope_split_q(_p(qn), _p(qr), _p(q), P, off, _p(inv_freq), _p(positions), T, H, D, Dr, rot_dims,
+                              int(bool(interleaved)), float(mag), _f32(q), _stream()), "rope_split_q")
     return qn, qr
+
+
+def head_gate(o: torch.Tensor, gate_src: Optional[torch.Tensor], g_off: int = 0) -> torch.Tensor:
+    """o [H, T, Dv] (a batched per-head product) -> [T, H * Dv], head h times sigmoid(gate_src[t, g_off + h])
+    (gate_src None: the layout change only)."""
+    if _ref(o):
+        return ref.head_gate(o, gate_src, g_off)
+    lib = require_mixers()
+    H, T, Dv = o.shape
+    assert o.is_contiguous()
+    gs = 0
+    if gate_src is not None:
+        assert gate_src.dtype == o.dtype and gate_src.is_contiguous() and gate_src.shape[0] >= T
+        gs = gate_src.shape[1]
+        assert 0 <= g_off and g_off + H <= gs
+    out = torch.empty((T, H * Dv), dtype=o.dtype, device=o.device)
+    check(lib.ka_head_gate(_p(out), _p(o), _p(gate_src), gs, g_off, T, H, Dv, _f32(o), _stream()), "head_gate")
+    return out
 
 
 def window_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor,
@@ -379,10 +422,11 @@ def window_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tens
 
 
 def moe_route(h: torch.Tensor, w_router: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int,
-              keep: int):
-    """-> (expert ids [T, top] int32, weights [T, top] fp32); see csrc/moe_route.hip."""
+              keep: int, sigmoid: bool = False, renorm: bool = True):
+    """-> (expert ids [T, top] int32, weights [T, top] fp32); see csrc/moe_route.hip.  sigmoid: the scores are the
+    logits' sigmoids instead of their softmax; renorm False: the weights are the chosen scores as they are."""
     if _ref(h):
-        return ref.moe_route(h, w_router, correction, top, groups, keep)
+        return ref.moe_route(h, w_router, correction, top, groups, keep, sigmoid, renorm)
     lib = require_mixers()
     T, W = h.shape
     E = w_router.shape[0]
@@ -390,18 +434,20 @@ def moe_route(h: torch.Tensor, w_router: torch.Tensor, correction: Optional[torc
     assert correction is None or (correction.dtype == torch.float32 and correction.numel() == E)
     ids = torch.empty((T, top), dtype=torch.int32, device=h.device)
     w = torch.empty((T, top), dtype=torch.float32, device=h.device)
-    check(lib.ka_moe_route(_p(ids), _p(w), _p(h), _p(w_router), _p(correction), T, W, E, top, groups, keep, _f32(h),
-                           _stream()), "moe_route")
+    check(lib.ka_moe_route(_p(ids), _p(w), _p(h), _p(w_router), _p(correction), T, W, E, top, groups, keep,
+                           int(bool(sigmoid)), int(bool(renorm)), _f32(h), _stream()), "moe_route")
     return ids, w
 
 
-def moe_experts(h: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+def moe_experts(h: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, w: torch.Tensor,
+                scale_input: bool = False) -> torch.Tensor:
     """sum_k w[t, k] * expert_{ids[t, k]}(h[t]) -> [T, W] fp32; w_gu [E, 2 ff, W] (gate rows, then up rows),
-    w_down [E, W, ff].  Decode-sized steps: in bf16 the rows grouped by expert on the matrix cores, otherwise
+    w_down [E, W, ff].  scale_input: sum_k expert_{ids[t, k]}(w[t, k] * h[t]) instead (the weight enters before the
+    expert's nonlinearity; it is applied to the fp32 results of the gate and up projections, which are linear).  Decode-sized steps: in bf16 the rows grouped by expert on the matrix cores, otherwise
     matrix-vector kernels straight from the stacked weights; neither reads the host, both are capturable.  More: rows sorted by expert, one read of the per-expert counts, one vendor GEMM pair per
     expert segment, weighted scatter-add in fp32."""
     if _ref(h):
-        return ref.moe_experts(h, w_gu, w_down, ids, w)
+        return ref.moe_experts(h, w_gu, w_down, ids, w, scale_input)
     T, W = h.shape
     E, two_ff, _ = w_gu.shape
     ff, top = two_ff // 2, ids.shape[1]
@@ -413,7 +459,7 @@ def moe_experts(h: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor, ids: 
         act = torch.empty((T * top, ff), dtype=h.dtype, device=h.device)
         yk = torch.empty((T * top, W), dtype=torch.float32, device=h.device)
         check(lib.ka_moe_grouped(_p(out), _p(act), _p(yk), _p(h), _p(w_gu), _p(w_down), _p(ids), _p(w), T, W, ff, top, E,
-                                 _stream()), "moe_grouped")
+                                 int(bool(scale_input)), _stream()), "moe_grouped")
         return out
     rows_ok = W * 4 <= 60 * 1024 and top * ff * 4 <= 60 * 1024 and top <= 32
     capturing = torch.cuda.is_current_stream_capturing()     # a graph cannot hold the sorted path's host read
@@ -422,8 +468,8 @@ def moe_experts(h: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor, ids: 
     if rows_ok and (capturing or T * top <= MOE_ROWS_MAX):
         lib = require_mixers()
         act = torch.empty((T * top, ff), dtype=h.dtype, device=h.device)
-        check(lib.ka_moe_rows(_p(out), _p(act), _p(h), _p(w_gu), _p(w_down), _p(ids), _p(w), T, W, ff, top, _f32(h),
-                              _stream()), "moe_rows")
+        check(lib.ka_moe_rows(_p(out), _p(act), _p(h), _p(w_gu), _p(w_down), _p(ids), _p(w), T, W, ff, top,
+                              int(bool(scale_input)), _f32(h), _stream()), "moe_rows")
         return out
     flat = ids.reshape(-1).long()
     order = torch.argsort(flat, stable=True)
@@ -431,12 +477,14 @@ def moe_experts(h: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor, ids: 
     tok = torch.div(order, top, rounding_mode="floor")
     xs = h.index_select(0, tok)
     ys = torch.empty((xs.shape[0], W), dtype=h.dtype, device=h.device)
+    ws = w.reshape(-1).index_select(0, order).contiguous()
     off = 0
     for e, c in enumerate(counts):
         if c:
-            ys[off:off + c] = F.linear(silu_mul(F.linear(xs[off:off + c], w_gu[e])), w_down[e])
+            gu = F.linear(xs[off:off + c], w_gu[e])
+            ys[off:off + c] = F.linear(silu_mul(gu, ws[off:off + c] if scale_input else None), w_down[e])
             off += c
-    out.index_add_(0, tok, ys.float() * w.reshape(-1).index_select(0, order).unsqueeze(1))
+    out.index_add_(0, tok, ys.float() if scale_input else ys.float() * ws.unsqueeze(1))
     return out
 
 
@@ -559,12 +607,14 @@ def short_conv(proj: torch.Tensor, off: int, C: int, w: torch.Tensor, state: Opt
 
 def rope_append(qkv: torch.Tensor, inv_freq: Optional[torch.Tensor], mag: float, positions: torch.Tensor,
                 slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, H: int, G: int, D: int, Dv: int,
-                rot: int) -> torch.Tensor:
-    """Rows [q (H x D) | k (G x D) | v (G x Dv)] -> q [T, H, D] with rotary positions on the first `rot` entries of
+                rot: int, q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None,
+                eps: float = 0.0) -> torch.Tensor:
+    """Rows [q (H x D) | k (G x D) | v (G x Dv)] -> q [T, H, D]; with q_norm / k_norm [D] fp32 every q / k head is
+    first divided by its root mean square (eps inside the root) and multiplied by that weight; then rotary positions on the first `rot` entries of
     each head (pairs (i, i + rot/2), angle = position * inv_freq[i] in fp32, cos and sin times `mag`); the rotated
     keys and the values are appended to the paged cache [NB, G, BS, D] / [NB, G, Dv, BS] at `slots` (-1: skipped)."""
     if _ref(qkv):
-        return ref.rope_append(qkv, inv_freq, mag, positions, slots, k_cache, v_cache, H, G, D, Dv, rot)
+        return ref.rope_append(qkv, inv_freq, mag, positions, slots, k_cache, v_cache, H, G, D, Dv, rot, q_norm, k_norm, eps)
     lib = require_mixers()
     T = qkv.shape[0]
     assert qkv.is_contiguous() and qkv.shape[1] == (H + G) * D + G * Dv and k_cache.dtype == qkv.dtype == v_cache.dtype
@@ -572,9 +622,12 @@ def rope_append(qkv: torch.Tensor, inv_freq: Optional[torch.Tensor], mag: float,
     assert k_cache.is_contiguous() and v_cache.is_contiguous()
     assert positions.dtype == torch.int32 and slots.dtype == torch.int32 and positions.shape[0] >= T and slots.shape[0] >= T
     assert rot == 0 or (inv_freq.dtype == torch.float32 and inv_freq.numel() * 2 == rot and rot <= D)
+    for nw in (q_norm, k_norm):
+        assert nw is None or (nw.dtype == torch.float32 and nw.numel() == D and nw.is_contiguous())
     q = torch.empty((T, H, D), dtype=qkv.dtype, device=qkv.device)
     check(lib.ka_rope_append(_p(q), _p(qkv), _p(inv_freq), float(mag), _p(positions), _p(slots), _p(k_cache), _p(v_cache),
-                             T, H, G, D, Dv, rot, k_cache.shape[2], _f32(qkv), _stream()), "rope_append")
+                             T, H, G, D, Dv, rot, k_cache.shape[2], _p(q_norm), _p(k_norm), float(eps), _f32(qkv), _stream()),
+          "rope_append")
     return q
 
 
@@ -584,16 +637,18 @@ SLIDING_TILE = True   # bf16 prompt portions of sliding attention on the matrix 
 def sliding_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                       q_starts: Optional[torch.Tensor], positions: torch.Tensor, slots: torch.Tensor,
                       gate_src: Optional[torch.Tensor], g_off: int, window: int, keep_first: int, scale: float,
-                      max_q: int = 0, num_decode: int = 0) -> torch.Tensor:
+                      max_q: int = 0, num_decode: int = 0, dist: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Softmax attention with grouped keys / values over a paged cache (k_cache [NB, G, BS, D], v_cache
     [NB, G, Dv, BS]): the query at position p sees the keys j <= p with p - j < window or j < keep_first (window 0:
     all of 0 .. p; kept keys stay at their own positions).  Head h's result is multiplied by
     sigmoid(gate_src[t, g_off + h]) (gate_src None: no gate).  q [T, H, D] -> [T, H * Dv].
     q_starts None: row t is block-table row t (a decode step).  max_q: the longest run of rows of one sequence in a
-    varlen step (0: unknown), num_decode: its leading one-row sequences; they choose the kernel, not the result."""
+    varlen step (0: unknown), num_decode: its leading one-row sequences; they choose the kernel, not the result.
+    dist [3, H] fp32 = (r1, r2, pb) per head: no softmax; the weight of a visible key at distance p - j is
+    sigmoid(score - r1 ln(1 + r2 (p - j)) + pb), and the weights are not normalised over the keys."""
     if _ref(q):
         return ref.sliding_attention(q, k_cache, v_cache, block_tables, q_starts, positions, slots, gate_src, g_off,
-                                     window, keep_first, scale)
+                                     window, keep_first, scale, dist)
     lib = require_mixers()
     T, H, D = q.shape
     G, BS, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
@@ -608,9 +663,11 @@ def sliding_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         assert gate_src.dtype == q.dtype and gate_src.is_contiguous() and gate_src.shape[0] >= T
         gs = gate_src.shape[1]
         assert 0 <= g_off and g_off + H <= gs
+    assert dist is None or (dist.dtype == torch.float32 and dist.shape == (3, H) and dist.is_contiguous())
+
     def tail(rows):
         return (_p(positions), _p(slots), _p(gate_src), gs, g_off, rows, H, G, D, Dv, int(window), int(keep_first), BS,
-                block_tables.shape[1], float(scale), _f32(q))
+                block_tables.shape[1], float(scale), _p(dist), _f32(q))
 
     tile = SLIDING_TILE and q.dtype == torch.bfloat16 and lib.ka_sliding_attention_tile_ok(H, G, D, Dv, BS)
     if tile and q_starts is not None and max_q >= 8:

@@ -157,10 +157,12 @@ def group_rmsnorm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float, out
     return y.to(out_dtype or x.dtype)
 
 
-def post_norm_residual(resid, y, w_post, ls, w_next, groups: int, eps: float):
-    """resid += ls * gnorm(y; w_post) (in place, fp32); returns gnorm(resid; w_next) in y's dtype, or None."""
-    resid.add_(ls.float() * group_rmsnorm(y, w_post, groups, eps, torch.float32))
-    return group_rmsnorm(resid, w_next, groups, eps, y.dtype) if w_next is not None else None
+def post_norm_residual(resid, y, w_post, ls, w_next, groups: int, eps: float, out_dtype=None):
+    """resid += ls * gnorm(y; w_post) (in place, fp32; ls None: 1); returns gnorm(resid; w_next) in out_dtype (y's by
+    default), or None."""
+    n = group_rmsnorm(y, w_post, groups, eps, torch.float32)
+    resid.add_(ls.float() * n if ls is not None else n)
+    return group_rmsnorm(resid, w_next, groups, eps, out_dtype or y.dtype) if w_next is not None else None
 
 
 def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
@@ -332,42 +334,63 @@ def headnorm_gate(o, proj, g_off: int, w, H: int, Dv: int, eps: float, out_dtype
     return (y * (F.silu(g) if silu else torch.sigmoid(g))).to(out_dtype)
 
 
-def _rot(x, positions, inv_freq, dims: int):
+def _rot(x, positions, inv_freq, dims: int, interleaved: bool = False, mag: float = 1.0):
+    """Rotary positions on the first `dims` entries: pairs (i, i + dims/2), or (2i, 2i + 1) when interleaved;
+    cos and sin times `mag`."""
     half = dims // 2
     if half == 0:
         return x
     ang = positions.float()[:, None] * inv_freq.float()[None, :]
     shape = [x.shape[0]] + [1] * (x.dim() - 2) + [half]
-    c, s = torch.cos(ang).view(shape), torch.sin(ang).view(shape)
+    c, s = (torch.cos(ang) * mag).view(shape), (torch.sin(ang) * mag).view(shape)
+    if interleaved:
+        a, b = x[..., 0:dims:2], x[..., 1:dims:2]
+        turned = torch.stack([a * c - b * s, b * c + a * s], dim=-1).flatten(-2)
+        return torch.cat([turned, x[..., dims:]], dim=-1)
     a, b = x[..., :half], x[..., half:dims]
     return torch.cat([a * c - b * s, b * c + a * s, x[..., dims:]], dim=-1)
 
 
-def latent_prep(proj, Q: int, R: int, Dr: int, w_q, w_kv, inv_freq, positions, slots, cache, rot_dims: int, eps: float):
+def latent_prep(proj, Q: int, R: int, Dr: int, w_q, w_kv, inv_freq, positions, slots, cache, rot_dims: int, eps: float,
+                interleaved: bool = False, mag: float = 1.0):
     """proj rows = [query latent Q | key/value latent R | rotated key part Dr] (the last two only with a cache).
-    -> the RMS-normed query latent [T, Q]; the normed latent and the rotated key part go to cache[slot]."""
-    cq = proj[:, :Q].float()
-    cq = (cq / torch.sqrt((cq * cq).mean(-1, keepdim=True) + eps) * w_q.float()).to(proj.dtype)
+    -> the RMS-normed query latent [T, Q] (None when Q is 0); the normed latent and the rotated key part go to
+    cache[slot]."""
+    cq = None
+    if Q:
+        cq = proj[:, :Q].float()
+        cq = (cq / torch.sqrt((cq * cq).mean(-1, keepdim=True) + eps) * w_q.float()).to(proj.dtype).contiguous()
     if cache is not None:
         c = proj[:, Q:Q + R].float()
         c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * w_kv.float()
-        kr = _rot(proj[:, Q + R:Q + R + Dr].float(), positions[:proj.shape[0]], inv_freq, rot_dims)
+        kr = _rot(proj[:, Q + R:Q + R + Dr].float(), positions[:proj.shape[0]], inv_freq, rot_dims, interleaved, mag)
         row = torch.cat([c, kr], dim=1).to(cache.dtype)
         s = slots[:proj.shape[0]].long()
         ok = s >= 0
         if ok.any():
             bs = cache.shape[1]
             cache[s[ok] // bs, s[ok] % bs] = row[ok]
-    return cq.contiguous()
+    return cq
 
 
-def rope_split_q(q, inv_freq, positions, H: int, D: int, Dr: int, rot_dims: int):
-    """q [T, H * (D + Dr)] -> (unrotated parts [H, T, D] in q's dtype, rotated parts [T, H, Dr] fp32)."""
+def rope_split_q(q, inv_freq, positions, H: int, D: int, Dr: int, rot_dims: int, interleaved: bool = False,
+                 mag: float = 1.0, off: int = 0):
+    """The columns off .. off + H * (D + Dr) of q's rows -> (unrotated parts [H, T, D] in q's dtype, rotated parts
+    [T, H, Dr] fp32)."""
     T = q.shape[0]
-    qh = q.view(T, H, D + Dr)
+    qh = q[:, off:off + H * (D + Dr)].reshape(T, H, D + Dr)
     qn = qh[:, :, :D].transpose(0, 1).contiguous()
-    qr = _rot(qh[:, :, D:].float(), positions[:T], inv_freq, rot_dims).contiguous()
+    qr = _rot(qh[:, :, D:].float(), positions[:T], inv_freq, rot_dims, interleaved, mag).contiguous()
     return qn, qr
+
+
+def head_gate(o, gate_src, g_off: int):
+    """o [H, T, Dv] -> [T, H * Dv], head h times sigmoid(gate_src[t, g_off + h]) (gate_src None: the layout only)."""
+    H, T, Dv = o.shape
+    y = o.transpose(0, 1).float()
+    if gate_src is not None:
+        y = y * torch.sigmoid(gate_src[:T, g_off:g_off + H].float())[:, :, None]
+    return y.reshape(T, H * Dv).to(o.dtype).contiguous()
 
 
 def window_attention(q_lat, q_rot, cache, block_tables, q_starts, positions, slots, sink, window: int, scale: float):
@@ -396,11 +419,13 @@ def window_attention(q_lat, q_rot, cache, block_tables, q_starts, positions, slo
     return out
 
 
-def moe_route(h, w_router, correction, top: int, groups: int, keep: int):
-    """Softmax scores over all experts; the choice adds `correction` and is limited to the `keep` groups (of
-    `groups` equal groups of neighbours) whose best choice score is largest; weights = the chosen experts'
-    scores (without correction) over their sum.  -> (ids [T, top] int32, weights [T, top] fp32)."""
-    s = torch.softmax(h.float() @ w_router.float().t(), dim=-1)
+def moe_route(h, w_router, correction, top: int, groups: int, keep: int, sigmoid: bool = False, renorm: bool = True):
+    """Scores over all experts (softmax of the router logits, or their sigmoids); the choice adds `correction` and is
+    limited to the `keep` groups (of `groups` equal groups of neighbours) whose best choice score is largest;
+    weights = the chosen experts' scores (without correction), over their sum when renorm.
+    -> (ids [T, top] int32, weights [T, top] fp32)."""
+    z = h.float() @ w_router.float().t()
+    s = torch.sigmoid(z) if sigmoid else torch.softmax(z, dim=-1)
     choice = s + correction.float() if correction is not None else s.clone()
     T, E = s.shape
     if groups > 1:
@@ -409,19 +434,38 @@ def moe_route(h, w_router, correction, top: int, groups: int, keep: int):
         choice = choice.masked_fill(~kept.repeat_interleave(E // groups, dim=1), float("-inf"))
     ids = torch.topk(choice, top, dim=-1).indices
     w = s.gather(1, ids)
-    return ids.to(torch.int32), w / (w.sum(-1, keepdim=True) + 1e-20)
+    return ids.to(torch.int32), (w / (w.sum(-1, keepdim=True) + 1e-20) if renorm else w.contiguous())
 
 
-def moe_experts(h, w_gu, w_down, ids, w) -> torch.Tensor:
+def silu_mul_scaled(gu: torch.Tensor, row_scale: torch.Tensor) -> torch.Tensor:
+    """silu(s g) * (s u) per row with its scale s: the gated unit of an input that was multiplied by s."""
+    g, u = gu.float().chunk(2, dim=-1)
+    sc = row_scale.float()[:, None]
+    return (F.silu(g * sc) * (u * sc)).to(gu.dtype)
+
+
+def moe_experts(h, w_gu, w_down, ids, w, scale_input: bool = False) -> torch.Tensor:
     """sum_k w[t, k] * down_e(silu(gate_e h) * up_e h), e = ids[t, k]; w_gu [E, 2 ff, W] = gate rows then up
-    rows, w_down [E, W, ff].  -> [T, W] fp32."""
+    rows, w_down [E, W, ff].  scale_input: the weight multiplies the expert's input instead,
+    sum_k down_e(silu(gate_e (w h)) * up_e (w h)), applied to the two projections' fp32 results.  -> [T, W] fp32."""
     T, W = h.shape
     out = torch.zeros((T, W), dtype=torch.float32, device=h.device)
     for e in torch.unique(ids).tolist():
         tok, slot = torch.nonzero(ids == e, as_tuple=True)
-        y = F.linear(silu_mul(F.linear(h[tok], w_gu[e])), w_down[e])
-        out.index_add_(0, tok, y.float() * w[tok, slot][:, None])
+        gu = F.linear(h[tok], w_gu[e])
+        if scale_input:
+            out.index_add_(0, tok, F.linear(silu_mul_scaled(gu, w[tok, slot]), w_down[e]).float())
+        else:
+            out.index_add_(0, tok, F.linear(silu_mul(gu), w_down[e]).float() * w[tok, slot][:, None])
     return out
+
+
+def glu_clamp(gu: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    """[T, 2 ff] = gate | up -> g sigmoid(alpha g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit)."""
+    g, u = gu.float().chunk(2, dim=-1)
+    g = g.clamp(max=limit)
+    u = u.clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -487,13 +531,19 @@ def short_conv(proj, off: int, C: int, w, state, seq_slots, q_starts, positions,
     return out
 
 
-def rope_append(qkv, inv_freq, mag: float, positions, slots, k_cache, v_cache, H: int, G: int, D: int, Dv: int, rot: int):
-    """Rows [q (H x D) | k (G x D) | v (G x Dv)]: rotary positions (angle = position * inv_freq, cos and sin times
-    mag) on the first `rot` entries of every q and k head; -> q [T, H, D]; k and v go to the paged cache
-    [NB, G, BS, D] / [NB, G, Dv, BS] at `slots`."""
+def rope_append(qkv, inv_freq, mag: float, positions, slots, k_cache, v_cache, H: int, G: int, D: int, Dv: int, rot: int,
+                q_norm=None, k_norm=None, eps: float = 0.0):
+    """Rows [q (H x D) | k (G x D) | v (G x Dv)]: with q_norm / k_norm [D], every q / k head is first divided by its
+    root mean square (eps inside the root) and multiplied by that weight; rotary positions (angle = position *
+    inv_freq, cos and sin times mag) on the first `rot` entries of every q and k head; -> q [T, H, D]; k and v go to
+    the paged cache [NB, G, BS, D] / [NB, G, Dv, BS] at `slots`."""
     T = qkv.shape[0]
     q = qkv[:, :H * D].float().view(T, H, D)
     k = qkv[:, H * D:(H + G) * D].float().view(T, G, D)
+    if q_norm is not None:
+        q = q / torch.sqrt((q * q).mean(-1, keepdim=True) + eps) * q_norm.float()
+    if k_norm is not None:
+        k = k / torch.sqrt((k * k).mean(-1, keepdim=True) + eps) * k_norm.float()
     v = qkv[:, (H + G) * D:(H + G) * D + G * Dv].view(T, G, Dv)
     half = rot // 2
     if half:
@@ -515,9 +565,10 @@ def rope_append(qkv, inv_freq, mag: float, positions, slots, k_cache, v_cache, H
 
 
 def sliding_attention(q, k_cache, v_cache, block_tables, q_starts, positions, slots, gate_src, g_off: int, window: int,
-                      keep_first: int, scale: float):
+                      keep_first: int, scale: float, dist=None):
     """q [T, H, D] -> [T, H * Dv]: softmax attention over the keys j <= p with p - j < window or j < keep_first
-    (window 0: all); head h's result times sigmoid(gate_src[t, g_off + h]) (gate_src None: no gate)."""
+    (window 0: all); head h's result times sigmoid(gate_src[t, g_off + h]) (gate_src None: no gate).
+    dist [3, H] = (r1, r2, pb): no softmax, a visible key's weight is sigmoid(score - r1 ln(1 + r2 (p - j)) + pb)."""
     T, H, D = q.shape
     G, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
     rep = H // G
@@ -533,7 +584,13 @@ def sliding_attention(q, k_cache, v_cache, block_tables, q_starts, positions, sl
             pages = block_tables[i].long()[js // bs]
             k = k_cache[pages, :, js % bs, :].float().repeat_interleave(rep, dim=1)   # [n, H, D]
             v = v_cache[pages, :, :, js % bs].float().repeat_interleave(rep, dim=1)   # [n, H, Dv]
-            w = torch.softmax(torch.einsum("hd,nhd->hn", q[t].float(), k) * scale, dim=1)
+            sc = torch.einsum("hd,nhd->hn", q[t].float(), k) * scale
+            if dist is not None:
+                d = (p - js).float()[None, :]
+                w = torch.sigmoid(sc - dist[0].float()[:, None] * torch.log1p(dist[1].float()[:, None] * d)
+                                  + dist[2].float()[:, None])
+            else:
+                w = torch.softmax(sc, dim=1)
             o = torch.einsum("hn,nhd->hd", w, v)
             if gate_src is not None:
                 o = o * torch.sigmoid(gate_src[t, g_off:g_off + H].float())[:, None]
