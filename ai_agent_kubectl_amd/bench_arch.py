@@ -7,7 +7,10 @@ with the same width, heads, head size, feed-forward width, vocabulary and depth 
 width ff/4 with 2 chosen plus a shared one, two residual streams), and with `...,suvapel` a Suvapel of that width and
 depth (layers alternating a delta rule with attention beside a channel-decay delta rule, window = the chunk, four
 taps, a 64-wide token input; its closest existing model is Kafilorn: recurrent state slots + windowed attention +
-fp32 residual), go through the same engine path (`build_engine`, the scheduler, `ModelRunner.execute`, hipGraph decode):
+fp32 residual), and with `...,zibinex` a Zibinex of that width and depth (gated latent attention and sliding sigmoid
+attention in turn, latent rank W/8 with a rotated part of half a head, the window = the chunk, the first layer's
+feed-forward dense and clamped, the others 8 experts of width ff/4 with 2 chosen; its closest existing model is Kafilorn:
+latent attention + experts + fp32 residual), go through the same engine path (`build_engine`, the scheduler, `ModelRunner.execute`, hipGraph decode):
 B prompts of P tokens are prefilled (in steps of the engine's token budget), then N tokens are
 decoded per sequence.  Reported per model: prefill tokens/s (prompt tokens / time in prefill steps)
 and decode tokens/s (B x decode steps / time in decode steps), from the runner's own step timers.
@@ -28,7 +31,7 @@ SIZES = {
 def _configs(size: str, chunk: int):
     import dataclasses
 
-    from .models.config import PRESETS, ModelConfig, kafilorn_uniform, suvapel_uniform, vivepel_uniform
+    from .models.config import PRESETS, ModelConfig, kafilorn_uniform, suvapel_uniform, vivepel_uniform, zibinex_uniform
 
     W, H, G, D, ff, V, L = SIZES[size]
     ll = ModelConfig(f"llama-{size}-{L}l", "llama", L, W, H, G, D, ff, V, 500000.0)
@@ -37,8 +40,11 @@ def _configs(size: str, chunk: int):
                           window=chunk, streams=2, kv_rank=W // 8, q_rank=3 * W // 8, dim=D, rot_dim=D // 2)
     kk = dataclasses.replace(kk, layers=kk.layers[:L])
     ss = suvapel_uniform(f"suvapel-{size}-{L}l", L, W, H, G, D, ff, V, window=chunk)
-    PRESETS[ll.name], PRESETS[vv.name], PRESETS[kk.name], PRESETS[ss.name] = ll, vv, kk, ss
-    return ll, vv, kk, ss
+    zz = zibinex_uniform(f"zibinex-{size}-{L}l", L, W, H, G, D, ff, V, window=chunk, kv_rank=W // 8, rot_dim=D // 2,
+                         experts=8, top=2, expert_ff=ff // 4)
+    for c in (ll, vv, kk, ss, zz):
+        PRESETS[c.name] = c
+    return ll, vv, kk, ss, zz
 
 
 def run_one(model: str, batch: int, prompt: int, new_tokens: int, warmup: int = 1, device: str = "cuda") -> dict:
@@ -84,8 +90,8 @@ def main(sizes=("2k", "8b"), batch: int = 32, prompt: int = 1024, new_tokens: in
          which=("llama", "vivepel")) -> dict:
     rows = []
     for size in sizes:
-        ll, vv, kk, ss = _configs(size, chunk)
-        for cfg in [c for c, n in ((ll, "llama"), (vv, "vivepel"), (kk, "kafilorn"), (ss, "suvapel")) if n in which]:
+        ll, vv, kk, ss, zz = _configs(size, chunk)
+        for cfg in [c for c, n in ((ll, "llama"), (vv, "vivepel"), (kk, "kafilorn"), (ss, "suvapel"), (zz, "zibinex")) if n in which]:
             r = run_one(cfg.name, batch, prompt, new_tokens)
             r["size"] = size
             rows.append(r)
@@ -103,4 +109,8 @@ def main(sizes=("2k", "8b"), batch: int = 32, prompt: int = 1024, new_tokens: in
               for s in sizes if (s, "suvapel") in by and (s, "kafilorn") in by}
     if sratio:
         out["suvapel_over_kafilorn"] = sratio
+    zratio = {s: {k: round(by[(s, "zibinex")][k] / by[(s, "kafilorn")][k], 3) for k in ("prefill_tok_s", "decode_tok_s")}
+              for s in sizes if (s, "zibinex") in by and (s, "kafilorn") in by}
+    if zratio:
+        out["zibinex_over_kafilorn"] = zratio
     return out

@@ -139,7 +139,7 @@ def parse_args(argv=None):
     ap.add_argument("--arch-batch", type=int, default=32)
     ap.add_argument("--arch-prompt", type=int, default=1024)
     ap.add_argument("--arch-chunk", type=int, default=1024, help="--arch-compare: Vivepel's attention chunk")
-    ap.add_argument("--arch-models", default="llama,vivepel", help="--arch-compare: of llama, vivepel, kafilorn, suvapel")
+    ap.add_argument("--arch-models", default="llama,vivepel", help="--arch-compare: of llama, vivepel, kafilorn, suvapel, zibinex")
     args = ap.parse_args(argv)
     if args.tp < 1 or args.gpus % args.tp:
         ap.error(f"--tp {args.tp} must divide --gpus {args.gpus}")

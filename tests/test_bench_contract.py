@@ -138,11 +138,13 @@ def test_arch_compare_is_an_option_and_off_by_default():
     b = bench.parse_args(["--arch-compare", "--arch-sizes", "2k"])
     assert b.arch_compare is True and b.arch_sizes == "2k"
     from ai_agent_kubectl_amd import bench_arch
-    ll, vv, kk, ss = bench_arch._configs("2k", 512)
+    ll, vv, kk, ss, zz = bench_arch._configs("2k", 512)
     assert (ll.hidden, ll.num_heads, ll.intermediate) == (vv.hidden, vv.layers[0].mixer.heads, vv.layers[0].ff)
     assert vv.layers[0].mixer.chunk == 512 and vv.num_layers == ll.num_layers
     assert (kk.hidden, kk.num_layers, kk.layers[0].mixer.heads) == (ll.hidden, ll.num_layers, ll.num_heads)
     assert kk.layers[1].mixer.window == 512 and kk.layers[2].mixer.kv_from == 1 and kk.layers[0].mlp.ff == ll.intermediate
     assert (ss.hidden, ss.num_layers, ss.layers[0].delta.heads, ss.layers[1].ff) == (ll.hidden, ll.num_layers, ll.num_heads, ll.intermediate)
     assert ss.layers[1].attention.window == 512 and ss.layers[0].attention is None and ss.layers[1].delta.channel_decay
-    assert b.arch_models == "llama,vivepel"          # Kafilorn and Suvapel join the comparison only when asked for
+    assert (zz.hidden, zz.num_layers, zz.layers[0].mixer.heads, zz.layers[0].mlp.ff) == (ll.hidden, ll.num_layers, ll.num_heads, ll.intermediate)
+    assert zz.layers[1].mixer.window == 512 and zz.layers[0].mixer.kind == "latent_attention" and zz.layers[1].mlp.kind == "moe"
+    assert b.arch_models == "llama,vivepel"          # Kafilorn, Suvapel and Zibinex join the comparison only when asked for

