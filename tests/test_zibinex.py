@@ -728,7 +728,7 @@ def test_sigmoid_attention_matrix_core_kernel(H, G, D, Dv, window):
                 outs.append(got.float().cpu())
         finally:
             mixers.SLIDING_TILE = True
-    assert (outs[0] - outs[3]).abs().max() < 3e-2
+    assert torch.allclose(outs[0], outs[3], rtol=1e-2, atol=3e-2)     # the two kernels: a bf16 rounding of the unnormalised sums apart
 
 
 @pytest.mark.gpu
