@@ -133,32 +133,32 @@ __global__ __launch_bounds__(512) void sliding_tile_kernel(bf16_t* __restrict__ 
       }
     }
     if constexpr (!SIG) {
-    mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-    const float m_new = fmaxf(m_run, mt);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;          // a query that has seen no key yet
-    const float corr = m_run == -INFINITY ? 1.f : __expf(m_run - m_use);
-    m_run = m_new;
-    float psum = 0.f;
+      mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      const float m_new = fmaxf(m_run, mt);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;          // a query that has seen no key yet
+      const float corr = m_run == -INFINITY ? 1.f : __expf(m_run - m_use);
+      m_run = m_new;
+      float psum = 0.f;
 #pragma unroll
-    for (int u = 0; u < NP; ++u)
+      for (int u = 0; u < NP; ++u)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float e = sv[u][r] == -INFINITY ? 0.f : __expf(sv[u][r] - m_use);
-        sv[u][r] = e;
-        psum += e;
+        for (int r = 0; r < 4; ++r) {
+          const float e = sv[u][r] == -INFINITY ? 0.f : __expf(sv[u][r] - m_use);
+          sv[u][r] = e;
+          psum += e;
+        }
+      l_run = l_run * corr + psum;
+      if (!__all(corr == 1.f)) {
+        float cr[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, 4 * grp + r, 64);
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) O[db][r] *= cr[r];
       }
-    l_run = l_run * corr + psum;
-    if (!__all(corr == 1.f)) {
-      float cr[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, 4 * grp + r, 64);
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) O[db][r] *= cr[r];
     }
-    }   // !SIG
 #pragma unroll
     for (int u = 0; u < NP; ++u) {
       if (i0 + u < total) {
