@@ -666,7 +666,7 @@ def suvapel_uniform(name: str, layers: int, hidden: int, heads: int, kv_heads: i
 
 # ------------------------------------------------------------------------------------------------
 # Zibinex: layers listed one by one, each x += norm(mixer(norm x)) then x += norm(ff(norm x)) with RMS norms whose
-# weights are stored around zero; a layer's mixer is latent attention with direct queries, interleaved YaRN-scaled
+# checkpoint weights are offsets from 1; a layer's mixer is latent attention with direct queries, interleaved YaRN-scaled
 # rotary positions and a sigmoid gate per head on the output, or sliding-window attention whose weights are
 # sigmoids of the score minus a logarithmic distance bias (no softmax); its feed-forward is a clamped gated unit,
 # a mixture of experts with a sigmoid router whose weight scales the expert's input, or absent.  A layer may run on

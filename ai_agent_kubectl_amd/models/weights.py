@@ -691,7 +691,7 @@ def load_suvapel_safetensors(path: str, cfg, device="cpu", dtype=torch.bfloat16)
 # ------------------------------------------------------------------------------------------------
 # Zibinex.  Engine layout per layer that has tensors of its own, `layers.<i>.` (activation dtype unless marked fp32;
 # a layer with weights_of has no entries, the model points it at its owner's):
-#   norm1, norm1b, norm2, norm2b [W] fp32, stored as 1 + w (the checkpoint keeps the weights around zero)
+#   norm1, norm1b, norm2, norm2b [W] fp32, kept as 1 + w (the checkpoint holds w, the offset from 1)
 #   latent attention:  w_in [dkv rows (kv_rank + rot_dim); q rows (H * (dim + rot_dim)); g rows (H); zero rows up to a
 #           multiple of 8, W] (one GEMM; `zibinex_columns`), kv_norm [kv_rank] fp32, w_uk [H, dim, kv_rank],
 #           w_uv [H, vdim, kv_rank], inv_freq [rot dims / 2] fp32 (YaRN-scaled, float64 rounded once), wo [W, H * vdim]

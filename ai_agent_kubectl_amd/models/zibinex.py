@@ -1,7 +1,7 @@
 """Zibinex decoder over the engine ops (`ops/mixers.py`).
 
 The residual x [T, W] is fp32.  A layer is x += n1b(mixer(n1(x))), then (if it has one) x += n2b(ff(n2(x))), every
-n an RMS norm x / sqrt(mean(x^2) + eps) * (1 + w) whose stored weight is around zero (the loader keeps 1 + w in fp32):
+n an RMS norm x / sqrt(mean(x^2) + eps) * (1 + w), w being what the checkpoint holds (the loader keeps 1 + w in fp32):
   h = norm(x)                                   group_rmsnorm with one group / fused into the update before it
   x += norm(y); h = next norm(x)                post_norm_residual (no layer scale)
 

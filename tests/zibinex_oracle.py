@@ -2,7 +2,7 @@
 token with no cache, written from the design's equations and sharing no code with the package.  Also the builders
 of small configurations and random checkpoints that the tests use.
 
-  norm(x; w)         x / sqrt(mean(x^2) + eps) * (1 + w)                      stored weights are around zero
+  norm(x; w)         x / sqrt(mean(x^2) + eps) * (1 + w)                      a checkpoint holds w, the offset from 1
   layer              x <- x + norm(mixer(norm(x; n1)); n1b);   x <- x + norm(ff(norm(x; n2)); n2b)
   latent attention   q_h = [q_h^n | q_h^r] rows of Wq h;  [c' | k^r] = Wdkv h;  c = c' / rms(c') * w_c
                      rotary on q_h^r and k^r, pairs (2i, 2i + 1), angle p f_i, cos and sin times a magnitude
