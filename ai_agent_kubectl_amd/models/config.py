@@ -708,6 +708,10 @@ class GatedLatentAttentionSpec:
     def cache_entries(self) -> int:
         return self.kv_rank + self.rot_dim
 
+    def tensor_sizes(self) -> tuple:
+        """What fixes the shapes of the mixer's tensors."""
+        return (self.kind, self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank)
+
 
 @dataclasses.dataclass(frozen=True)
 class SigmoidAttentionSpec:
@@ -740,6 +744,10 @@ class SigmoidAttentionSpec:
     def cache_entries(self) -> int:
         return self.kv_heads * (self.dim + self.vdim)
 
+    def tensor_sizes(self) -> tuple:
+        """What fixes the shapes of the mixer's tensors."""
+        return (self.kind, self.heads, self.kv_heads, self.dim, self.vdim)
+
 
 @dataclasses.dataclass(frozen=True)
 class ClampedFeedForwardSpec:
@@ -770,12 +778,17 @@ class ClampedFeedForwardSpec:
             return {"kind": "dense", "ff": self.ff, "limit": self.limit}
         return {"kind": "moe", "expert": {"ff": self.ff}, "router": {"experts": self.experts, "top": self.top}}
 
+    def tensor_sizes(self) -> tuple:
+        """What fixes the shapes of the feed-forward's tensors."""
+        return (self.kind, self.ff, self.experts)
+
 
 @dataclasses.dataclass(frozen=True)
 class ZibinexLayer:
     mixer: object               # GatedLatentAttentionSpec | SigmoidAttentionSpec
     mlp: Optional[ClampedFeedForwardSpec]
-    weights_of: int = -1        # >= 0: no tensors of its own, runs on that layer's; its cache is its own
+    weights_of: int = -1        # >= 0: no tensors of its own, runs on that layer's; its cache is its own, and so are the
+                                # constants of its entry (window, scale, rotation, limit, top)
 
 
 _ZIBINEX_MIXERS = {"latent_attention": GatedLatentAttentionSpec, "attention": SigmoidAttentionSpec}
@@ -816,7 +829,8 @@ class ZibinexConfig:
         for i, L in enumerate(layers):
             if L.weights_of >= 0:
                 src = layers[L.weights_of] if L.weights_of < len(layers) and L.weights_of != i else None
-                if src is None or src.weights_of >= 0 or (src.mixer, src.mlp) != (L.mixer, L.mlp):
+                sizes = lambda l: (l.mixer.tensor_sizes(), l.mlp.tensor_sizes() if l.mlp is not None else None)
+                if src is None or src.weights_of >= 0 or sizes(src) != sizes(L):
                     raise ValueError(f"layer {i}: weights_of {L.weights_of} must name another layer of the same sizes "
                                      "that has tensors of its own")
         return cls(name=name, vocab_size=int(d["vocab"]), hidden=int(d["width"]), norm_eps=float(d["norm"]["eps"]),

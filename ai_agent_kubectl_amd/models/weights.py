@@ -694,13 +694,13 @@ def load_suvapel_safetensors(path: str, cfg, device="cpu", dtype=torch.bfloat16)
 #   norm1, norm1b, norm2, norm2b [W] fp32, kept as 1 + w (the checkpoint holds w, the offset from 1)
 #   latent attention:  w_in [dkv rows (kv_rank + rot_dim); q rows (H * (dim + rot_dim)); g rows (H); zero rows up to a
 #           multiple of 8, W] (one GEMM; `zibinex_columns`), kv_norm [kv_rank] fp32, w_uk [H, dim, kv_rank],
-#           w_uv [H, vdim, kv_rank], inv_freq [rot dims / 2] fp32 (YaRN-scaled, float64 rounded once), wo [W, H * vdim]
+#           w_uv [H, vdim, kv_rank], wo [W, H * vdim] (the rotary table belongs to the layer's entry: the model makes it)
 #   attention:  w_qkv [q; k; v rows, W] + b_qkv (one GEMM), q_norm / k_norm [dim] fp32, dist [3, H] fp32 (the rows
 #           r1, r2, pb), wo [W, H * vdim]
 #   dense feed-forward:  w_gu [gate rows; up rows, W], w_down [W, ff]
 #   experts:  w_router [E, W] fp32, w_gu_e [E, 2 ff, W] (gate rows, then up rows), w_dn_e [E, W, ff]
 # The LM head is the embedding table.
-_ZIBINEX_F32 = ("norm1", "norm1b", "norm2", "norm2b", "kv_norm", "inv_freq", "q_norm", "k_norm", "dist", "w_router")
+_ZIBINEX_F32 = ("norm1", "norm1b", "norm2", "norm2b", "kv_norm", "q_norm", "k_norm", "dist", "w_router")
 
 
 def zibinex_columns(m) -> Dict[str, int]:
@@ -728,7 +728,6 @@ def _zibinex_pack(cfg, get, device, dtype) -> Dict[str, torch.Tensor]:
             W[p + "kv_norm"] = get(c + "mix.dkv.norm")
             W[p + "w_uk"] = get(c + "mix.uk").view(m.heads, m.dim, m.kv_rank)
             W[p + "w_uv"] = get(c + "mix.uv").view(m.heads, m.vdim, m.kv_rank)
-            W[p + "inv_freq"] = torch.tensor(m.rot.frequencies()[0], dtype=torch.float64)
         else:
             W[p + "w_qkv"] = torch.cat([get(c + "mix.q"), get(c + "mix.k"), get(c + "mix.v")])
             W[p + "b_qkv"] = torch.cat([get(c + "mix.q.b"), get(c + "mix.k.b"), get(c + "mix.v.b")])
@@ -763,8 +762,7 @@ def zibinex_check_shapes(cfg, W: Dict[str, torch.Tensor]) -> None:
         want.update({p + "norm1": (h,), p + "norm1b": (h,), p + "wo": (h, m.heads * m.vdim)})
         if m.kind == "latent_attention":
             want.update({p + "w_in": (zibinex_columns(m)["total"], h), p + "kv_norm": (m.kv_rank,),
-                         p + "w_uk": (m.heads, m.dim, m.kv_rank), p + "w_uv": (m.heads, m.vdim, m.kv_rank),
-                         p + "inv_freq": (m.rot.dims // 2,)})
+                         p + "w_uk": (m.heads, m.dim, m.kv_rank), p + "w_uv": (m.heads, m.vdim, m.kv_rank)})
         else:
             n = m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)
             want.update({p + "w_qkv": (n, h), p + "b_qkv": (n,), p + "q_norm": (m.dim,), p + "k_norm": (m.dim,),

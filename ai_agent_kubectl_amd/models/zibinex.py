@@ -21,7 +21,8 @@ Feed-forwards: dense down(g sigmoid(1.702 g) (u + 1)), g = min(gate h, limit), u
 or experts chosen by a sigmoid router (moe_route: sigmoid scores, no renormalisation) whose score multiplies the
 expert's input, summed in fp32 (moe_experts with scale_input).
 
-A layer with `weights_of` runs on its owner's tensors (the same dict) with a cache of its own.  Cache: per layer
+A layer with `weights_of` runs on its owner's tensors (the same dict) with a cache of its own and the constants of
+its own entry (window, scale, rotary table, limit, top).  Cache: per layer
 either the latent rows [NB, BS, kv_rank + rot_dim] or K [NB, G, BS, D] and V [NB, G, Dv, BS], under the engine's single
 block table.  No recurrent state.  Prefill, chunked prefill, mixed and decode steps all run this forward; the decode
 step is shape-static and capturable.
@@ -56,15 +57,18 @@ class ZibinexModel:
         self.vocab_offset = 0
         own: Dict[int, dict] = {}
         for i, spec in enumerate(cfg.layers):
-            if spec.weights_of >= 0:
-                continue
-            p = f"layers.{i}."
-            L = {k[len(p):]: v for k, v in weights.items() if k.startswith(p)}
-            if spec.mixer.kind == "latent_attention":
-                L["rot_mag"] = spec.mixer.rot.frequencies()[1]   # YaRN's factor on cos and sin (1 without scaling)
-                L["cols"] = zibinex_columns(spec.mixer)
-            own[i] = L
+            if spec.weights_of < 0:
+                p = f"layers.{i}."
+                own[i] = {k[len(p):]: v for k, v in weights.items() if k.startswith(p)}
         self.layers: List[dict] = [own[cfg.owner(i)] for i in range(cfg.num_layers)]
+        # per layer, from its own entry: the rotary table (frequencies in float64 rounded once to fp32; the angle is
+        # position * frequency in fp32), YaRN's factor on cos and sin (1 without scaling), the fused row's columns
+        self.rotary: List[Optional[tuple]] = [None] * cfg.num_layers
+        for i, spec in enumerate(cfg.layers):
+            if spec.mixer.kind == "latent_attention":
+                f, mag = spec.mixer.rot.frequencies()
+                inv = torch.tensor(f, dtype=torch.float64).to(device=self.device, dtype=torch.float32)
+                self.rotary[i] = (inv, mag, zibinex_columns(spec.mixer))
         # the runner's hooks shared with LlamaModel
         self.persistent = False
         self.mark_layer = -1
@@ -100,12 +104,12 @@ class ZibinexModel:
         return 0
 
     # ---- sublayers -----------------------------------------------------------------------------
-    def _latent_attention(self, h, L, m, cache, meta: AttnMeta):
-        col, mag, eps = L["cols"], L["rot_mag"], self.cfg.norm_eps
+    def _latent_attention(self, h, L, m, li, cache, meta: AttnMeta):
+        (inv_freq, mag, col), eps = self.rotary[li], self.cfg.norm_eps
         proj = F.linear(h, L["w_in"])                                  # [T, c | k_r | q | g]
-        mixers.latent_prep(proj, 0, m.kv_rank, m.rot_dim, None, L["kv_norm"], L["inv_freq"], meta.positions,
+        mixers.latent_prep(proj, 0, m.kv_rank, m.rot_dim, None, L["kv_norm"], inv_freq, meta.positions,
                            meta.slot_mapping, cache, m.rot.dims, eps, interleaved=True, mag=mag)
-        qn, qr = mixers.rope_split_q(proj, L["inv_freq"], meta.positions, m.heads, m.dim, m.rot_dim, m.rot.dims,
+        qn, qr = mixers.rope_split_q(proj, inv_freq, meta.positions, m.heads, m.dim, m.rot_dim, m.rot.dims,
                                      interleaved=True, mag=mag, off=col["q"])
         q_lat = torch.bmm(qn, L["w_uk"])                               # [H, T, R]
         o_lat = mixers.window_attention(q_lat, qr, cache, meta.block_tables, None if meta.is_decode else meta.q_starts,
@@ -141,7 +145,7 @@ class ZibinexModel:
                 self.mark_event.record()
             m, f = spec.mixer, spec.mlp
             if m.kind == "latent_attention":
-                y = self._latent_attention(h, L, m, k_cache[li], meta)
+                y = self._latent_attention(h, L, m, li, k_cache[li], meta)
             else:
                 y = self._attention(h, L, m, k_cache[li], v_cache[li], meta)
             nxt = self.layers[li + 1]["norm1"] if li < last else None

@@ -127,10 +127,15 @@ def variant(name):
     if name == "window_one":     # a window of one position (only the token itself), equal head counts, top 1
         return make_config([attention_layer(heads=2, kv_heads=2, dim=4, vdim=6, window=1, top=1),
                             attention_layer(heads=4, kv_heads=4, dim=5, vdim=3, window=17, mlp="dense")], width=12, vocab=32)
+    if name == "own_constants":  # layers on another's tensors whose entries differ in what is not a tensor's size: window, scale,
+        # rotary table, number of chosen experts
+        return make_config([attention_layer(window=8), latent_layer(),
+                            shared(attention_layer(window=3, scale=0.9, top=1), 0),
+                            shared(latent_layer(window=4, scaling=None, base=50.0, scale=0.2, top=3), 1)])
     raise KeyError(name)
 
 
-VARIANTS = ["base", "odd", "no_mask", "window_one"]
+VARIANTS = ["base", "odd", "no_mask", "window_one", "own_constants"]
 
 
 def model_for(tmp_path, name, seed=0, every_expert=False):
@@ -589,6 +594,7 @@ def test_config_reader(tmp_path):
                  lambda b: b["layers"][1]["mlp"].__setitem__("kind", "experts"),
                  lambda b: b["layers"][1]["mlp"]["router"].__setitem__("top", 9),     # more than there are experts
                  lambda b: b["layers"][4].__setitem__("weights_of", 1),               # another kind of layer
+                 lambda b: b["layers"][4]["mixer"].__setitem__("kv_rank", 10),        # other tensor sizes than its owner's
                  lambda b: b["layers"][4].__setitem__("weights_of", 4),               # itself
                  lambda b: b["layers"][2].__setitem__("weights_of", 4)):              # a layer that has none of its own
         bad = variant("base")

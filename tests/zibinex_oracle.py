@@ -14,7 +14,7 @@ of small configurations and random checkpoints that the tests use.
   dense              Wd (g sigmoid(1.702 g) (u + 1)),  g = min(Wg h, limit),  u = clamp(Wu h, -limit, limit)
   experts            s = sigmoid(Wr h);  the `top` largest s_e;  y = sum_e E_e(s_e h),  E(x) = Wd (silu(Wg x) * Wu x)
   logits             embed . norm(x; final)
-A layer with weights_of = j computes with layer j's tensors.
+A layer with weights_of = j computes with layer j's tensors and the constants of its own entry.
 """
 import math
 
@@ -203,7 +203,7 @@ def ff_cfg(kind, ff=20, limit=0.75, experts=5, top=2):
 
 
 def shared(layer, owner):
-    """A layer that runs on layer `owner`'s tensors (the rest of its entry equals the owner's)."""
+    """A layer that runs on layer `owner`'s tensors (the sizes of its entry equal the owner's)."""
     return dict(layer, weights_of=owner)
 
 
